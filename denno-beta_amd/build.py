@@ -42,6 +42,8 @@ LIBRARIES = {
                      "kernels/gemm_direct.hip"], ["kernels/common.h", "kernels/gemm_common.h"]),
     "attention": ("hip", ["kernels/attention.hip"], ["kernels/common.h", "kernels/attention.h"]),
     "sampling": ("hip", ["kernels/sampling.hip"], ["kernels/common.h"]),
+    "sequence": ("hip", ["kernels/sequence.hip"], ["kernels/common.h"]),
+    "grouped": ("hip", ["kernels/grouped.hip"], ["kernels/common.h"]),
 }
 
 _loaded = {}

@@ -2,7 +2,7 @@
 
 The reference dispatches on config.json's `model_type` and fails on an unknown one
 (crates/denno-engine/src/model/mod.rs:88-104).  Here the key is `architectures[0]`
-(what model folders name their class with), with `model_type` as the fallback.
+(what model folders name their class with), with `architecture` (one name) and `model_type` as the fallbacks.
 """
 from __future__ import annotations
 
@@ -41,8 +41,9 @@ def resolve_architecture(config_json: dict) -> Architecture:
     archs = config_json.get("architectures")
     if isinstance(archs, list):
         names += [a for a in archs if isinstance(a, str)]
-    if isinstance(config_json.get("model_type"), str):
-        names.append(config_json["model_type"])
+    for key in ("architecture", "model_type"):
+        if isinstance(config_json.get(key), str):
+            names.append(config_json[key])
     for n in names:
         if n in _BY_NAME:
             return _BY_NAME[n]
@@ -56,7 +57,20 @@ def load_config(model_dir: str):
     """-> (Architecture, typed config) of a model folder."""
     d = read_config_json(model_dir)
     arch = resolve_architecture(d)
-    return arch, arch.config_cls.from_dict(d)
+    cfg = arch.config_cls.from_dict(d)
+    if hasattr(cfg, "with_shapes"):
+        # an architecture whose config.json leaves a size to the tensors themselves reads it from the file's header
+        from ..weights.safetensors_io import SafetensorsError, open_checkpoint
+        try:
+            where, files = open_checkpoint(model_dir)
+        except (OSError, SafetensorsError):
+            return arch, cfg
+        try:
+            cfg = cfg.with_shapes({name: tuple(where[name].entries[name][1]) for name in where})
+        finally:
+            for f in files:
+                f.close()
+    return arch, cfg
 
 
 def _ensure_builtin():

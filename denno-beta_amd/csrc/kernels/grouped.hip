@@ -1,0 +1,287 @@
+// Products whose weight depends on the row's group: a matrix per head (out[t, h, :] = W_h a[t, h, :]) and a
+// matrix per expert for the rows that a router sent there.  One tile routine serves both: 16 rows x 64 columns a
+// workgroup of 256 threads, K in chunks of 32 through LDS, 32-bit sums in ascending order of k, so a row's result
+// does not depend on which other rows share its tile.  Also the router's choice and the plan that sorts a step's
+// (row, choice) pairs by expert.
+#include "common.h"
+
+namespace {
+
+__device__ __forceinline__ float load_as(const void* p, size_t i, int dt) {
+  return dt == DN_F32 ? static_cast<const float*>(p)[i] : to_float(static_cast<const bf16_t*>(p)[i]);
+}
+__device__ __forceinline__ void store_as(void* p, size_t i, int dt, float v) {
+  if (dt == DN_F32) static_cast<float*>(p)[i] = v;
+  else static_cast<bf16_t*>(p)[i] = from_float<bf16_t>(v);
+}
+
+constexpr int TM = 16, TN = 64, TK = 32;
+
+struct Tile {
+  float a[TM][TK + 1];
+  float w[TN][TK + 1];
+};
+
+// acc[c] (c < 4) += sum_k A[row, k] * W[n0 + cq * 4 + c, k] for this thread's row `tid / 16` and columns cq = tid % 16.
+// a_row[q]: element offset of row tid / 32 + 8 q of the tile in A, or -1 where the tile has no such row.
+// DUAL: a second weight W2 with its own sums.
+template <bool DUAL>
+__device__ __forceinline__ void tile_product(Tile& lds, Tile* lds2, const void* A, int a_dt, const long long a_row[2], const void* W,
+                                             const void* W2, int w_dt, size_t w_base, int N, int K, int n0, float acc[4],
+                                             float acc2[4]) {
+  const int tid = threadIdx.x;
+  const int lr = tid >> 5, lk = tid & 31;      // loads: row (or column of W) and k
+  const int r = tid >> 4, cq = tid & 15;       // sums
+  for (int k0 = 0; k0 < K; k0 += TK) {
+    const bool kin = k0 + lk < K;
+#pragma unroll
+    for (int q = 0; q < 2; ++q)
+      lds.a[lr + 8 * q][lk] = (kin && a_row[q] >= 0) ? load_as(A, static_cast<size_t>(a_row[q]) + k0 + lk, a_dt) : 0.f;
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {
+      const int n = n0 + lr + 8 * q;
+      const bool ok = kin && n < N;
+      const size_t at = w_base + static_cast<size_t>(n) * K + k0 + lk;
+      lds.w[lr + 8 * q][lk] = ok ? load_as(W, at, w_dt) : 0.f;
+      if (DUAL) lds2->w[lr + 8 * q][lk] = ok ? load_as(W2, at, w_dt) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < TK; ++kk) {
+      const float av = lds.a[r][kk];
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        acc[c] = fmaf(av, lds.w[cq * 4 + c][kk], acc[c]);
+        if (DUAL) acc2[c] = fmaf(av, lds2->w[cq * 4 + c][kk], acc2[c]);
+      }
+    }
+    __syncthreads();
+  }
+}
+
+// ---- a matrix per head ---------------------------------------------------------------------------------------
+// out[t, o_off + h * o_stride + n] = sum_k W[h][n][k] * a[t, a_off + h * a_stride + k]
+__global__ __launch_bounds__(256) void heads_linear_kernel(const void* A, int a_dt, size_t lda, int a_off, int a_stride, const void* W,
+                                                           int w_dt, void* out, int out_dt, size_t ldo, int o_off, int o_stride,
+                                                           int T, int N, int K) {
+  __shared__ Tile lds;
+  const int h = blockIdx.z, t0 = blockIdx.x * TM, n0 = blockIdx.y * TN;
+  const int tid = threadIdx.x;
+  long long a_row[2];
+#pragma unroll
+  for (int q = 0; q < 2; ++q) {
+    const int t = t0 + (tid >> 5) + 8 * q;
+    a_row[q] = t < T ? static_cast<long long>(t) * lda + a_off + static_cast<long long>(h) * a_stride : -1;
+  }
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};
+  tile_product<false>(lds, nullptr, A, a_dt, a_row, W, nullptr, w_dt, static_cast<size_t>(h) * N * K, N, K, n0, acc, nullptr);
+  const int t = t0 + (tid >> 4);
+  if (t >= T) return;
+#pragma unroll
+  for (int c = 0; c < 4; ++c) {
+    const int n = n0 + (tid & 15) * 4 + c;
+    if (n < N) store_as(out, static_cast<size_t>(t) * ldo + o_off + static_cast<size_t>(h) * o_stride + n, out_dt, acc[c]);
+  }
+}
+
+// ---- the router's choice -------------------------------------------------------------------------------------
+// Per row: s = softmax(z) over the experts; the `top` largest of s + correction are chosen (the lower index wins a
+// tie), weighed by their s divided by the sum of the chosen s (+ 1e-20).  A thread a row.
+__global__ __launch_bounds__(64) void route_kernel(const float* z, const float* correction, int T, int E, int top, int* ids, float* wts) {
+  const int t = blockIdx.x * 64 + threadIdx.x;
+  if (t >= T) return;
+  const float* row = z + static_cast<size_t>(t) * E;
+  float m = row[0];
+  for (int e = 1; e < E; ++e) m = fmaxf(m, row[e]);
+  float sum = 0.f;
+  for (int e = 0; e < E; ++e) sum += expf(row[e] - m);
+  float chosen_sum = 0.f;
+  for (int c = 0; c < top; ++c) {
+    int best = -1;
+    float best_v = 0.f, best_s = 0.f;
+    for (int e = 0; e < E; ++e) {
+      bool taken = false;
+      for (int q = 0; q < c; ++q) taken |= ids[t * top + q] == e;
+      if (taken) continue;
+      const float sc = expf(row[e] - m) / sum;
+      const float v = sc + (correction ? correction[e] : 0.f);
+      if (best < 0 || v > best_v) best = e, best_v = v, best_s = sc;
+    }
+    ids[t * top + c] = best;
+    wts[t * top + c] = best_s;
+    chosen_sum += best_s;
+  }
+  const float inv = 1.0f / (chosen_sum + 1e-20f);
+  for (int c = 0; c < top; ++c) wts[t * top + c] *= inv;
+}
+
+// ---- the plan ------------------------------------------------------------------------------------------------
+// The n pairs (row, choice), pair i = row * top + choice, sorted by expert and inside an expert by i:
+// offsets[e] .. offsets[e + 1] - 1 are expert e's places in `order`.  One workgroup.
+__global__ __launch_bounds__(256) void plan_kernel(const int* ids, int n, int E, int* offsets, int* order) {
+  extern __shared__ int shm[];
+  int* base = shm;         // [E]
+  int* cid = shm + E;      // [256]
+  const int tid = threadIdx.x;
+  for (int e = tid; e < E; e += 256) base[e] = 0;
+  __syncthreads();
+  for (int i = tid; i < n; i += 256) atomicAdd(&base[ids[i]], 1);
+  __syncthreads();
+  if (tid == 0) {
+    int run = 0;
+    for (int e = 0; e < E; ++e) {
+      const int c = base[e];
+      offsets[e] = run;
+      base[e] = run;
+      run += c;
+    }
+    offsets[E] = run;
+  }
+  __syncthreads();
+  for (int c0 = 0; c0 < n; c0 += 256) {
+    const int i = c0 + tid;
+    const int e = i < n ? ids[i] : -1;
+    cid[tid] = e;
+    __syncthreads();
+    if (e >= 0) {
+      int rank = 0;
+      for (int q = 0; q < tid; ++q) rank += cid[q] == e;
+      order[base[e] + rank] = i;
+    }
+    __syncthreads();
+    if (e >= 0) atomicAdd(&base[e], 1);
+    __syncthreads();
+  }
+}
+
+// which expert and which of its tiles of 16 places workgroup `id` has; false: none
+__device__ __forceinline__ bool expert_tile(const int* offsets, int E, int id, int& e, int& p0, int& p1) {
+  for (e = 0; e < E; ++e) {
+    const int cnt = offsets[e + 1] - offsets[e];
+    const int tiles = (cnt + TM - 1) / TM;
+    if (id < tiles) {
+      p0 = offsets[e] + id * TM;
+      p1 = min(p0 + TM, offsets[e + 1]);
+      return true;
+    }
+    id -= tiles;
+  }
+  return false;
+}
+
+// ---- an expert's first half: y[p, :] = g * sigmoid(alpha g) * (u + 1), g = min(W_gate h, limit), u = clamp(W_up h, +-limit) --
+__global__ __launch_bounds__(256) void expert_up_kernel(const void* h, int h_dt, size_t ldh, const int* order, const int* offsets,
+                                                        int E, int top, const void* wg, const void* wu, int w_dt, int ff, int width,
+                                                        float limit, float alpha, void* y, int y_dt) {
+  __shared__ Tile lds, lds2;
+  int e, p0, p1;
+  if (!expert_tile(offsets, E, blockIdx.x, e, p0, p1)) return;
+  const int tid = threadIdx.x, n0 = blockIdx.y * TN;
+  long long a_row[2];
+#pragma unroll
+  for (int q = 0; q < 2; ++q) {
+    const int p = p0 + (tid >> 5) + 8 * q;
+    a_row[q] = p < p1 ? static_cast<long long>(order[p] / top) * ldh : -1;
+  }
+  float g[4] = {0.f, 0.f, 0.f, 0.f}, u[4] = {0.f, 0.f, 0.f, 0.f};
+  tile_product<true>(lds, &lds2, h, h_dt, a_row, wg, wu, w_dt, static_cast<size_t>(e) * ff * width, ff, width, n0, g, u);
+  const int p = p0 + (tid >> 4);
+  if (p >= p1) return;
+#pragma unroll
+  for (int c = 0; c < 4; ++c) {
+    const int n = n0 + (tid & 15) * 4 + c;
+    if (n >= ff) continue;
+    const float gv = fminf(g[c], limit), uv = fminf(fmaxf(u[c], -limit), limit);
+    store_as(y, static_cast<size_t>(p) * ff + n, y_dt, gv / (1.0f + expf(-alpha * gv)) * (uv + 1.0f));
+  }
+}
+
+// ---- an expert's second half: out[pair, :] = W_down y[p, :] ------------------------------------------------------
+__global__ __launch_bounds__(256) void expert_down_kernel(const void* y, int y_dt, const int* order, const int* offsets, int E,
+                                                          const void* wd, int w_dt, int width, int ff, float* out) {
+  __shared__ Tile lds;
+  int e, p0, p1;
+  if (!expert_tile(offsets, E, blockIdx.x, e, p0, p1)) return;
+  const int tid = threadIdx.x, n0 = blockIdx.y * TN;
+  long long a_row[2];
+#pragma unroll
+  for (int q = 0; q < 2; ++q) {
+    const int p = p0 + (tid >> 5) + 8 * q;
+    a_row[q] = p < p1 ? static_cast<long long>(p) * ff : -1;
+  }
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};
+  tile_product<false>(lds, nullptr, y, y_dt, a_row, wd, nullptr, w_dt, static_cast<size_t>(e) * width * ff, width, ff, n0, acc, nullptr);
+  const int p = p0 + (tid >> 4);
+  if (p >= p1) return;
+  const size_t pair = order[p];
+#pragma unroll
+  for (int c = 0; c < 4; ++c) {
+    const int n = n0 + (tid & 15) * 4 + c;
+    if (n < width) out[pair * width + n] = acc[c];
+  }
+}
+
+// x[t, :] += sum_c wts[t, c] * out[t * top + c, :], the choices in their order
+__global__ __launch_bounds__(256) void combine_kernel(const float* out, const float* wts, int top, int width, float* x, size_t ldx) {
+  const int t = blockIdx.x;
+  for (int c = threadIdx.x; c < width; c += 256) {
+    float acc = 0.f;
+    for (int q = 0; q < top; ++q) acc = fmaf(wts[t * top + q], out[(static_cast<size_t>(t) * top + q) * width + c], acc);
+    x[t * ldx + c] += acc;
+  }
+}
+
+bool float_kind(int dt) { return dt == DN_F32 || dt == DN_BF16; }
+
+}  // namespace
+
+extern "C" {
+
+int dn_heads_linear(const void* a, int a_dt, long long lda, int a_off, int a_stride, const void* w, int w_dt, void* out, int out_dt,
+                    long long ldo, int o_off, int o_stride, int T, int H, int N, int K, hipStream_t stream) {
+  if (!float_kind(a_dt) || !float_kind(w_dt) || !float_kind(out_dt)) return DN_ERR_DTYPE;
+  if (H < 1 || N < 1 || K < 1 || H > 65535) return DN_ERR_SHAPE;
+  if (T == 0) return 0;
+  hipLaunchKernelGGL(heads_linear_kernel, dim3((T + TM - 1) / TM, (N + TN - 1) / TN, H), dim3(256), 0, stream, a, a_dt,
+                     static_cast<size_t>(lda), a_off, a_stride, w, w_dt, out, out_dt, static_cast<size_t>(ldo), o_off, o_stride, T, N, K);
+  return dn_launch_status();
+}
+
+int dn_moe_route(const float* z, const float* correction, int T, int E, int top, int* ids, float* wts, hipStream_t stream) {
+  if (E < 1 || top < 1 || top > E) return DN_ERR_SHAPE;
+  if (T == 0) return 0;
+  hipLaunchKernelGGL(route_kernel, dim3((T + 63) / 64), dim3(64), 0, stream, z, correction, T, E, top, ids, wts);
+  return dn_launch_status();
+}
+
+int dn_moe_plan(const int* ids, int n, int E, int* offsets, int* order, hipStream_t stream) {
+  if (E < 1 || E > 8192) return DN_ERR_SHAPE;
+  hipLaunchKernelGGL(plan_kernel, dim3(1), dim3(256), (E + 256) * sizeof(int), stream, ids, n, E, offsets, order);
+  return dn_launch_status();
+}
+
+int dn_moe_up(const void* h, int h_dt, long long ldh, const int* order, const int* offsets, int E, int top, int n, const void* wg,
+              const void* wu, int w_dt, int ff, int width, float limit, float alpha, void* y, int y_dt, hipStream_t stream) {
+  if (!float_kind(h_dt) || !float_kind(w_dt) || !float_kind(y_dt)) return DN_ERR_DTYPE;
+  if (n == 0) return 0;
+  hipLaunchKernelGGL(expert_up_kernel, dim3((n + TM - 1) / TM + E, (ff + TN - 1) / TN), dim3(256), 0, stream, h, h_dt,
+                     static_cast<size_t>(ldh), order, offsets, E, top, wg, wu, w_dt, ff, width, limit, alpha, y, y_dt);
+  return dn_launch_status();
+}
+
+int dn_moe_down(const void* y, int y_dt, const int* order, const int* offsets, int E, int n, const void* wd, int w_dt, int width,
+                int ff, float* out, hipStream_t stream) {
+  if (!float_kind(y_dt) || !float_kind(w_dt)) return DN_ERR_DTYPE;
+  if (n == 0) return 0;
+  hipLaunchKernelGGL(expert_down_kernel, dim3((n + TM - 1) / TM + E, (width + TN - 1) / TN), dim3(256), 0, stream, y, y_dt, order,
+                     offsets, E, wd, w_dt, width, ff, out);
+  return dn_launch_status();
+}
+
+int dn_moe_combine(const float* out, const float* wts, int T, int top, int width, float* x, long long ldx, hipStream_t stream) {
+  if (T == 0) return 0;
+  hipLaunchKernelGGL(combine_kernel, dim3(T), dim3(256), 0, stream, out, wts, top, width, x, static_cast<size_t>(ldx));
+  return dn_launch_status();
+}
+
+}  // extern "C"

@@ -1,0 +1,406 @@
+// Kernels for layers that carry something from token to token besides keys and values: norms without a
+// mean, short causal convolutions over time, the previous token's row, turned pairs of dimensions, and
+// matrix states that decay (one scan for every recurrence of the form S <- diag(w) S + a v^T).
+// Everything here is 32-bit arithmetic; only what is read or stored may be bfloat16.  A request's rows
+// are rows row_start[s] .. row_start[s + 1] - 1 of the step, its state lies at slots[s]; a request whose
+// slot is negative is padding and is skipped.
+#include "common.h"
+
+namespace {
+
+__device__ __forceinline__ float load_as(const void* p, size_t i, int dt) {
+  return dt == DN_F32 ? static_cast<const float*>(p)[i] : to_float(static_cast<const bf16_t*>(p)[i]);
+}
+__device__ __forceinline__ void store_as(void* p, size_t i, int dt, float v) {
+  if (dt == DN_F32) static_cast<float*>(p)[i] = v;
+  else static_cast<bf16_t*>(p)[i] = from_float<bf16_t>(v);
+}
+
+// the request that owns row t: the last s with row_start[s] <= t
+__device__ __forceinline__ int request_of(const int* row_start, int S, int t) {
+  int lo = 0, hi = S - 1;
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) >> 1;
+    if (row_start[mid] <= t) lo = mid; else hi = mid - 1;
+  }
+  return lo;
+}
+
+// sum over a workgroup of 256 threads, the same in every thread; waves are joined in order
+__device__ __forceinline__ float block_sum_256(float v, float* sh) {
+  v = wave_sum(v);
+  const int wave = threadIdx.x >> 6;
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) sh[wave] = v;
+  __syncthreads();
+  return (sh[0] + sh[1]) + (sh[2] + sh[3]);
+}
+
+// ---- norm without a mean -----------------------------------------------------------------------------------
+// out[r, :] = x[row, :width] / sqrt(mean(x^2) + eps) * weight; one workgroup a row; a thread sums its own
+// columns in ascending order, so a row's result does not depend on what else is in the step.
+__global__ __launch_bounds__(256) void rmsnorm_kernel(const void* x, int x_dt, size_t ldx, const float* weight, void* out,
+                                                      int out_dt, size_t ldo, const int* rows, int width, float eps) {
+  __shared__ float sh[4];
+  const int r = blockIdx.x;
+  const size_t src = static_cast<size_t>(rows ? rows[r] : r) * ldx;
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < width; c += 256) {
+    const float v = load_as(x, src + c, x_dt);
+    ss = fmaf(v, v, ss);
+  }
+  ss = block_sum_256(ss, sh);
+  const float inv = 1.0f / sqrtf(ss / static_cast<float>(width) + eps);
+  for (int c = threadIdx.x; c < width; c += 256) {
+    const float v = load_as(x, src + c, x_dt) * inv;
+    store_as(out, static_cast<size_t>(r) * ldo + c, out_dt, weight ? v * weight[c] : v);
+  }
+}
+
+// out[t, :] = [a[t, :wa] | b[t, :wb]]
+__global__ __launch_bounds__(256) void concat_kernel(const float* a, size_t lda, int wa, const float* b, size_t ldb, int wb,
+                                                     void* out, int out_dt) {
+  const int t = blockIdx.x;
+  const size_t o = static_cast<size_t>(t) * (wa + wb);
+  for (int c = threadIdx.x; c < wa + wb; c += 256)
+    store_as(out, o + c, out_dt, c < wa ? a[t * lda + c] : b[t * ldb + (c - wa)]);
+}
+
+// ---- short causal convolution over time ----------------------------------------------------------------------
+// out[t, c] = h[t, c] + sum_j w[c, j] * h[t - taps + 1 + j, c]; rows before the step's first row of a request come
+// from its history [slot][taps - 1][width] (oldest first; zero for a new request).
+__global__ __launch_bounds__(256) void conv_rows_kernel(const float* h, const float* w, const float* hist, const int* row_start,
+                                                        const int* slots, int S, int width, int taps, void* out, int out_dt, size_t hist_stride) {
+  const int t = blockIdx.x;
+  const int s = request_of(row_start, S, t);
+  const int slot = slots[s];
+  if (slot < 0) return;
+  const int i = t - row_start[s];
+  const float* past = hist + static_cast<size_t>(slot) * hist_stride;
+  for (int c = threadIdx.x; c < width; c += 256) {
+    float acc = h[static_cast<size_t>(t) * width + c];
+    for (int j = 0; j < taps; ++j) {
+      const int src = i - taps + 1 + j;
+      const float v = src >= 0 ? h[static_cast<size_t>(row_start[s] + src) * width + c] : past[static_cast<size_t>(i + j) * width + c];
+      acc = fmaf(w[c * taps + j], v, acc);
+    }
+    store_as(out, static_cast<size_t>(t) * width + c, out_dt, acc);
+  }
+}
+
+// The last `keep` rows of (history ++ this step's rows) become the history.  A thread owns a channel of a request and
+// goes through the places in ascending order: place m reads the old place m + n, which it has not written yet.
+__global__ __launch_bounds__(256) void history_update_kernel(const void* h, int h_dt, float* hist, const int* row_start,
+                                                             const int* slots, int width, int keep, size_t hist_stride) {
+  const int s = blockIdx.x;
+  const int slot = slots[s];
+  if (slot < 0) return;
+  const int row0 = row_start[s], n = row_start[s + 1] - row0;
+  float* past = hist + static_cast<size_t>(slot) * hist_stride;
+  for (int c = threadIdx.x; c < width; c += 256)
+    for (int m = 0; m < keep; ++m) {
+      const int src = n - keep + m;
+      past[static_cast<size_t>(m) * width + c] =
+          src >= 0 ? load_as(h, static_cast<size_t>(row0 + src) * width + c, h_dt) : past[static_cast<size_t>(m + n) * width + c];
+    }
+}
+
+// out[m][t][c] = h[t][c] + (h[t - 1][c] - h[t][c]) * mu[m][c]; the row before a request's first row of the step is
+// its history (one row a slot).
+__global__ __launch_bounds__(256) void shift_mix_kernel(const void* h, int h_dt, const float* hist, const float* mu, int n_mix,
+                                                        const int* row_start, const int* slots, int S, int T, int width,
+                                                        void* out, int out_dt, size_t hist_stride) {
+  const int t = blockIdx.x;
+  const int s = request_of(row_start, S, t);
+  const int slot = slots[s];
+  if (slot < 0) return;
+  const bool first = t == row_start[s];
+  for (int c = threadIdx.x; c < width; c += 256) {
+    const float cur = load_as(h, static_cast<size_t>(t) * width + c, h_dt);
+    const float prev = first ? hist[static_cast<size_t>(slot) * hist_stride + c] : load_as(h, static_cast<size_t>(t - 1) * width + c, h_dt);
+    const float d = prev - cur;
+    for (int m = 0; m < n_mix; ++m)
+      store_as(out, (static_cast<size_t>(m) * T + t) * width + c, out_dt, fmaf(d, mu[m * width + c], cur));
+  }
+}
+
+// ---- pairs of dimensions turned by the position ------------------------------------------------------------
+// Vector n of row t starts at src_off + n * src_stride; its entries 2i and 2i + 1 (i < dims / 2) are turned by the
+// angle position * freq[i], the other `width - dims` entries pass; the result goes to dst_off + n * dst_stride.
+__global__ __launch_bounds__(256) void rotary_kernel(const void* src, int src_dt, size_t ld_src, int src_off, int src_stride,
+                                                     void* dst, int dst_dt, size_t ld_dst, int dst_off, int dst_stride,
+                                                     const int* positions, const float* freq, int n_vec, int dims, int width) {
+  const int t = blockIdx.x;
+  const float p = static_cast<float>(positions[t]);
+  const int half = dims / 2, rest = width - dims;
+  const int per = half + rest;
+  for (int e = threadIdx.x; e < n_vec * per; e += 256) {
+    const int n = e / per, i = e % per;
+    const size_t a = static_cast<size_t>(t) * ld_src + src_off + static_cast<size_t>(n) * src_stride;
+    const size_t b = static_cast<size_t>(t) * ld_dst + dst_off + static_cast<size_t>(n) * dst_stride;
+    if (i < half) {
+      const float ang = p * freq[i];
+      const float c = cosf(ang), sn = sinf(ang);
+      const float u = load_as(src, a + 2 * i, src_dt), v = load_as(src, a + 2 * i + 1, src_dt);
+      store_as(dst, b + 2 * i, dst_dt, u * c - v * sn);
+      store_as(dst, b + 2 * i + 1, dst_dt, v * c + u * sn);
+    } else {
+      const int k = dims + (i - half);
+      store_as(dst, b + k, dst_dt, load_as(src, a + k, src_dt));
+    }
+  }
+}
+
+// ---- activations of projections that feed a recurrence or a gate --------------------------------------------
+enum { ACT_SILU = 0, ACT_SIGMOID = 1, ACT_TANH = 2, ACT_EXP_NEG_EXP = 3, ACT_BOUNDED_SIGMOID = 4 };
+
+__device__ __forceinline__ float sigmoid_f(float z) { return 1.0f / (1.0f + expf(-z)); }
+
+__device__ __forceinline__ float activation(int kind, float z, float lower) {
+  switch (kind) {
+    case ACT_SILU: return z * sigmoid_f(z);
+    case ACT_SIGMOID: return sigmoid_f(z);
+    case ACT_TANH: return tanhf(z);
+    case ACT_EXP_NEG_EXP: return expf(-expf(z));
+    default: return lower + (1.0f - lower) * sigmoid_f(z);
+  }
+}
+
+// out[t, c] = act(x[t, c] + bias[c]) (lower[c]: the least value of a bounded sigmoid)
+__global__ __launch_bounds__(256) void activate_kernel(const float* x, size_t ldx, const float* bias, const float* lower, int kind,
+                                                       void* out, int out_dt, size_t ldo, int n) {
+  const int t = blockIdx.x;
+  for (int c = threadIdx.x; c < n; c += 256) {
+    const float z = x[t * ldx + c] + (bias ? bias[c] : 0.f);
+    store_as(out, t * ldo + c, out_dt, activation(kind, z, lower ? lower[c] : 0.f));
+  }
+}
+
+// out[t, c] = x[t, c] * act(g[t, c])
+__global__ __launch_bounds__(256) void gated_kernel(const void* x, int x_dt, size_t ldx, const float* g, size_t ldg, int kind,
+                                                    void* out, int out_dt, size_t ldo, int n) {
+  const int t = blockIdx.x;
+  for (int c = threadIdx.x; c < n; c += 256)
+    store_as(out, t * ldo + c, out_dt, load_as(x, t * ldx + c, x_dt) * activation(kind, g[t * ldg + c], 0.f));
+}
+
+// ---- the scan ----------------------------------------------------------------------------------------------
+// Per request, head and value column j a lane keeps column j of the head's state S [dk][dv] in registers and walks
+// the request's rows of this step in order:
+//   a_i = key_from_decay ? 1 - w_i : k_i
+//   read_after:   S_i <- w_i S_i + a_i v_j ;  o_j = sum_i r_i S_i
+//   else:         o_j = sum_i r_i (S_i + u_i a_i v_j) ;  S_i <- w_i S_i + a_i v_j
+// The sum over i runs in ascending order, one fused multiply-add a step, whatever the step holds.  A row's r, k and w
+// reach the lanes through LDS; the next row's are asked for before the current row is worked on.
+struct ScanArgs {
+  const float *r, *k, *v, *w, *u;
+  size_t ldr, ldk, ldv, ldw;
+  float* state;
+  size_t slot_stride;
+  const int *row_start, *slots;
+  int H, dk, dv, read_after, key_from_decay;
+  float* out;
+  size_t ldo;
+};
+
+template <int DK>
+__global__ __launch_bounds__(64) void scan_kernel(ScanArgs a) {
+  constexpr int NL = DK >= 64 ? DK / 64 : 1;
+  __shared__ float sh[3 * DK];
+  __shared__ float shu[DK];
+  const int s = blockIdx.z, h = blockIdx.y, lane = threadIdx.x;
+  const int j = blockIdx.x * 64 + lane;
+  const int slot = a.slots[s];
+  if (slot < 0) return;
+  const int row0 = a.row_start[s], row1 = a.row_start[s + 1];
+  if (row0 >= row1) return;
+  const bool live = j < a.dv;
+  const int dk = a.dk, dv = a.dv;
+  float* sp = a.state + static_cast<size_t>(slot) * a.slot_stride + static_cast<size_t>(h) * dk * dv + j;
+  float S[DK];
+#pragma unroll
+  for (int i = 0; i < DK; ++i) S[i] = (live && i < dk) ? sp[static_cast<size_t>(i) * dv] : 0.f;
+  for (int i = lane; i < DK; i += 64) shu[i] = (a.u && i < dk) ? a.u[h * dk + i] : 0.f;
+  float nr[NL], nk[NL], nw[NL], nv;
+  auto fetch = [&](int t) {
+#pragma unroll
+    for (int q = 0; q < NL; ++q) {
+      const int i = lane + 64 * q;
+      const bool ok = i < dk;
+      nr[q] = ok ? a.r[t * a.ldr + h * dk + i] : 0.f;
+      nk[q] = (ok && !a.key_from_decay) ? a.k[t * a.ldk + h * dk + i] : 0.f;
+      nw[q] = ok ? a.w[t * a.ldw + h * dk + i] : 1.f;
+    }
+    nv = live ? a.v[t * a.ldv + h * dv + j] : 0.f;
+  };
+  fetch(row0);
+  for (int t = row0; t < row1; ++t) {
+#pragma unroll
+    for (int q = 0; q < NL; ++q) {
+      const int i = lane + 64 * q;
+      if (i < DK) {
+        sh[i] = nr[q];
+        sh[DK + i] = a.key_from_decay ? 1.0f - nw[q] : nk[q];
+        sh[2 * DK + i] = nw[q];
+      }
+    }
+    const float vj = nv;
+    __syncthreads();
+    if (t + 1 < row1) fetch(t + 1);
+    float o = 0.f;
+    if (a.read_after) {
+#pragma unroll
+      for (int i = 0; i < DK; ++i) {
+        S[i] = fmaf(sh[2 * DK + i], S[i], sh[DK + i] * vj);
+        o = fmaf(sh[i], S[i], o);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < DK; ++i) {
+        const float kv = sh[DK + i] * vj;
+        o = fmaf(sh[i], fmaf(shu[i], kv, S[i]), o);
+        S[i] = fmaf(sh[2 * DK + i], S[i], kv);
+      }
+    }
+    if (live) a.out[t * a.ldo + h * dv + j] = o;
+    __syncthreads();
+  }
+  if (live)
+#pragma unroll
+    for (int i = 0; i < DK; ++i)
+      if (i < dk) sp[static_cast<size_t>(i) * dv] = S[i];
+}
+
+// ---- a norm per head, with a gate ----------------------------------------------------------------------------
+// out[t, h, j] = o[t, h, j] / sqrt(mean_j(o^2) + eps) * weight[h * w_stride + j] * act(gate[t, h, j]); a wave a head.
+__global__ __launch_bounds__(64) void head_norm_kernel(const float* o, size_t ld, const float* weight, int w_stride, float eps,
+                                                       const float* gate, size_t ldg, int gate_kind, void* out, int out_dt,
+                                                       size_t ldo, int dv) {
+  const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const float* src = o + t * ld + static_cast<size_t>(h) * dv;
+  float ss = 0.f;
+  for (int j = lane; j < dv; j += 64) ss = fmaf(src[j], src[j], ss);
+  ss = wave_sum(ss);
+  const float inv = 1.0f / sqrtf(ss / static_cast<float>(dv) + eps);
+  for (int j = lane; j < dv; j += 64) {
+    float y = src[j] * inv;
+    if (weight) y *= weight[h * w_stride + j];
+    if (gate) y *= activation(gate_kind, gate[t * ldg + static_cast<size_t>(h) * dv + j], 0.f);
+    store_as(out, t * ldo + static_cast<size_t>(h) * dv + j, out_dt, y);
+  }
+}
+
+bool float_kind(int dt) { return dt == DN_F32 || dt == DN_BF16; }
+
+}  // namespace
+
+extern "C" {
+
+int dn_rmsnorm(const void* x, int x_dt, long long ldx, const float* weight, void* out, int out_dt, long long ldo, const int* rows,
+               int R, int width, float eps, hipStream_t stream) {
+  if (!float_kind(x_dt) || !float_kind(out_dt)) return DN_ERR_DTYPE;
+  if (R < 0 || width < 1) return DN_ERR_SHAPE;
+  if (R == 0) return 0;
+  hipLaunchKernelGGL(rmsnorm_kernel, dim3(R), dim3(256), 0, stream, x, x_dt, static_cast<size_t>(ldx), weight, out, out_dt,
+                     static_cast<size_t>(ldo), rows, width, eps);
+  return dn_launch_status();
+}
+
+int dn_concat_cast(const float* a, long long lda, int wa, const float* b, long long ldb, int wb, void* out, int out_dt, int T,
+                   hipStream_t stream) {
+  if (!float_kind(out_dt)) return DN_ERR_DTYPE;
+  if (T == 0) return 0;
+  hipLaunchKernelGGL(concat_kernel, dim3(T), dim3(256), 0, stream, a, static_cast<size_t>(lda), wa, b, static_cast<size_t>(ldb), wb,
+                     out, out_dt);
+  return dn_launch_status();
+}
+
+int dn_conv_rows(const float* h, const float* w, const float* hist, const int* row_start, const int* slots, int S, int T, int width,
+                 int taps, void* out, int out_dt, long long hist_stride, hipStream_t stream) {
+  if (!float_kind(out_dt)) return DN_ERR_DTYPE;
+  if (taps < 1 || S < 1) return DN_ERR_SHAPE;
+  if (T == 0) return 0;
+  hipLaunchKernelGGL(conv_rows_kernel, dim3(T), dim3(256), 0, stream, h, w, hist, row_start, slots, S, width, taps, out, out_dt,
+                     static_cast<size_t>(hist_stride));
+  return dn_launch_status();
+}
+
+int dn_history_update(const void* h, int h_dt, float* hist, const int* row_start, const int* slots, int S, int width, int keep,
+                      long long hist_stride, hipStream_t stream) {
+  if (!float_kind(h_dt)) return DN_ERR_DTYPE;
+  if (S == 0 || keep == 0) return 0;
+  hipLaunchKernelGGL(history_update_kernel, dim3(S), dim3(256), 0, stream, h, h_dt, hist, row_start, slots, width, keep,
+                     static_cast<size_t>(hist_stride));
+  return dn_launch_status();
+}
+
+int dn_shift_mix(const void* h, int h_dt, const float* hist, const float* mu, int n_mix, const int* row_start, const int* slots, int S,
+                 int T, int width, void* out, int out_dt, long long hist_stride, hipStream_t stream) {
+  if (!float_kind(h_dt) || !float_kind(out_dt)) return DN_ERR_DTYPE;
+  if (S < 1) return DN_ERR_SHAPE;
+  if (T == 0) return 0;
+  hipLaunchKernelGGL(shift_mix_kernel, dim3(T), dim3(256), 0, stream, h, h_dt, hist, mu, n_mix, row_start, slots, S, T, width, out,
+                     out_dt, static_cast<size_t>(hist_stride));
+  return dn_launch_status();
+}
+
+int dn_rotary(const void* src, int src_dt, long long ld_src, int src_off, int src_stride, void* dst, int dst_dt, long long ld_dst,
+              int dst_off, int dst_stride, const int* positions, const float* freq, int T, int n_vec, int dims, int width,
+              hipStream_t stream) {
+  if (!float_kind(src_dt) || !float_kind(dst_dt)) return DN_ERR_DTYPE;
+  if (dims % 2 != 0 || dims > width || dims < 0) return DN_ERR_SHAPE;
+  if (T == 0 || n_vec == 0) return 0;
+  hipLaunchKernelGGL(rotary_kernel, dim3(T), dim3(256), 0, stream, src, src_dt, static_cast<size_t>(ld_src), src_off, src_stride, dst,
+                     dst_dt, static_cast<size_t>(ld_dst), dst_off, dst_stride, positions, freq, n_vec, dims, width);
+  return dn_launch_status();
+}
+
+int dn_activate(const float* x, long long ldx, const float* bias, const float* lower, int kind, void* out, int out_dt, long long ldo,
+                int T, int n, hipStream_t stream) {
+  if (!float_kind(out_dt)) return DN_ERR_DTYPE;
+  if (kind < 0 || kind > ACT_BOUNDED_SIGMOID) return DN_ERR_SHAPE;
+  if (T == 0) return 0;
+  hipLaunchKernelGGL(activate_kernel, dim3(T), dim3(256), 0, stream, x, static_cast<size_t>(ldx), bias, lower, kind, out, out_dt,
+                     static_cast<size_t>(ldo), n);
+  return dn_launch_status();
+}
+
+int dn_gated(const void* x, int x_dt, long long ldx, const float* g, long long ldg, int kind, void* out, int out_dt, long long ldo,
+             int T, int n, hipStream_t stream) {
+  if (!float_kind(x_dt) || !float_kind(out_dt)) return DN_ERR_DTYPE;
+  if (kind < 0 || kind > ACT_TANH) return DN_ERR_SHAPE;
+  if (T == 0) return 0;
+  hipLaunchKernelGGL(gated_kernel, dim3(T), dim3(256), 0, stream, x, x_dt, static_cast<size_t>(ldx), g, static_cast<size_t>(ldg), kind,
+                     out, out_dt, static_cast<size_t>(ldo), n);
+  return dn_launch_status();
+}
+
+int dn_state_scan(const float* r, long long ldr, const float* k, long long ldk, const float* v, long long ldv, const float* w,
+                  long long ldw, const float* u, float* state, long long slot_stride, const int* row_start, const int* slots, int S,
+                  int H, int dk, int dv, int read_after, int key_from_decay, float* out, long long ldo, hipStream_t stream) {
+  if (dk < 1 || dk > 256 || dv < 1 || H < 1) return DN_ERR_SHAPE;
+  if (!key_from_decay && k == nullptr) return DN_ERR_SHAPE;
+  if (S == 0) return 0;
+  ScanArgs a{r, k, v, w, u, static_cast<size_t>(ldr), static_cast<size_t>(ldk), static_cast<size_t>(ldv), static_cast<size_t>(ldw),
+             state, static_cast<size_t>(slot_stride), row_start, slots, H, dk, dv, read_after, key_from_decay, out,
+             static_cast<size_t>(ldo)};
+  const dim3 grid((dv + 63) / 64, H, S);
+  if (dk <= 16) hipLaunchKernelGGL(scan_kernel<16>, grid, dim3(64), 0, stream, a);
+  else if (dk <= 32) hipLaunchKernelGGL(scan_kernel<32>, grid, dim3(64), 0, stream, a);
+  else if (dk <= 64) hipLaunchKernelGGL(scan_kernel<64>, grid, dim3(64), 0, stream, a);
+  else if (dk <= 128) hipLaunchKernelGGL(scan_kernel<128>, grid, dim3(64), 0, stream, a);
+  else hipLaunchKernelGGL(scan_kernel<256>, grid, dim3(64), 0, stream, a);
+  return dn_launch_status();
+}
+
+int dn_head_norm(const float* o, long long ld, const float* weight, int w_stride, float eps, const float* gate, long long ldg,
+                 int gate_kind, void* out, int out_dt, long long ldo, int T, int H, int dv, hipStream_t stream) {
+  if (!float_kind(out_dt)) return DN_ERR_DTYPE;
+  if (gate && (gate_kind < 0 || gate_kind > ACT_TANH)) return DN_ERR_SHAPE;
+  if (T == 0) return 0;
+  hipLaunchKernelGGL(head_norm_kernel, dim3(T, H), dim3(64), 0, stream, o, static_cast<size_t>(ld), weight, w_stride, eps, gate,
+                     static_cast<size_t>(ldg), gate_kind, out, out_dt, static_cast<size_t>(ldo), dv);
+  return dn_launch_status();
+}
+
+}  // extern "C"

@@ -35,7 +35,8 @@ class ModelRunner:
             from ..build import ensure_built
             from ..parts.base import PagedKV
             paged = any(isinstance(cs, PagedKV) for cs in model.cache_specs)
-            ensure_built(["host", "elementwise", "gemm"] + (["attention"] if paged else []))
+            more = sorted({lib for p in model.all_parts() for lib in getattr(p, "libraries", ())})
+            ensure_built(["host", "elementwise", "gemm"] + (["attention"] if paged else []) + more)
         self.model = model.bind(tensors, self.runtime)
         cache_tokens = options.cache_tokens or options.max_live * spec.max_positions
         self.cache = CacheStorage(self.model.cache_specs, kv_dtype=self.runtime.act_dtype,

@@ -122,6 +122,27 @@ def _declare(name, lib):
             "dn_attention_flash": [P, I, P, I, P, P, P, I, P, P, P, P, I, I, I, I, I, F, I, P],
             "dn_attention_decode": [P, I, P, I, P, P, P, I, P, P, P, I, P, I, I, I, I, I, I, I, F, I, P],
         },
+        "sequence": {
+            "dn_rmsnorm": [P, I, c_longlong, P, P, I, c_longlong, P, I, I, F, P],
+            "dn_concat_cast": [P, c_longlong, I, P, c_longlong, I, P, I, I, P],
+            "dn_conv_rows": [P, P, P, P, P, I, I, I, I, P, I, c_longlong, P],
+            "dn_history_update": [P, I, P, P, P, I, I, I, c_longlong, P],
+            "dn_shift_mix": [P, I, P, P, I, P, P, I, I, I, P, I, c_longlong, P],
+            "dn_rotary": [P, I, c_longlong, I, I, P, I, c_longlong, I, I, P, P, I, I, I, I, P],
+            "dn_activate": [P, c_longlong, P, P, I, P, I, c_longlong, I, I, P],
+            "dn_gated": [P, I, c_longlong, P, c_longlong, I, P, I, c_longlong, I, I, P],
+            "dn_state_scan": [P, c_longlong, P, c_longlong, P, c_longlong, P, c_longlong, P, P, c_longlong, P, P, I, I, I, I, I, I,
+                              P, c_longlong, P],
+            "dn_head_norm": [P, c_longlong, P, I, F, P, c_longlong, I, P, I, c_longlong, I, I, I, P],
+        },
+        "grouped": {
+            "dn_heads_linear": [P, I, c_longlong, I, I, P, I, P, I, c_longlong, I, I, I, I, I, I, P],
+            "dn_moe_route": [P, P, I, I, I, P, P, P],
+            "dn_moe_plan": [P, I, I, P, P, P],
+            "dn_moe_up": [P, I, c_longlong, P, P, I, I, I, P, P, I, I, I, F, F, P, I, P],
+            "dn_moe_down": [P, I, P, P, I, I, P, I, I, I, P, P],
+            "dn_moe_combine": [P, P, I, I, I, P, c_longlong, P],
+        },
         "sampling": {
             "dn_sample": [P, I, I, I, P, P, P, P],
             "dn_penalties": [P, I, I, I, P, P, P, P, P, P, P, P],
@@ -886,3 +907,259 @@ def linear_norm_in(copy, stats, c1, c2, eps, w, out, epilogue="none", kv=None, n
         "linear_norm_in" if _timed is None else
         f"norm + linear {K} -> {N}" + (", cache write" if kv is not None else "") + (f", {epilogue}" if epilogue != "none" else ""))
     return out if kv is None else out[:, :kv[3]]
+
+
+# -- layers that carry more than keys and values from token to token (csrc/kernels/sequence.hip) -----------------------
+ACTIVATIONS = {"silu": 0, "sigmoid": 1, "tanh": 2, "exp_neg_exp": 3, "bounded_sigmoid": 4}
+
+
+def _f32vec(t, name, n=None):
+    if t is None:
+        return None
+    _dev(t, name, (torch.float32,))
+    _need(t.is_contiguous() and (n is None or t.numel() == n), lambda: f"{name}: {tuple(t.shape)}, wanted {n} contiguous 32-bit numbers")
+    return t
+
+
+def _request_tables(row_start, slots, what):
+    _dev(row_start, "row_start", _I32, 1), _dev(slots, "slots", _I32, 1)
+    S = slots.shape[0]
+    _need(row_start.is_contiguous() and slots.is_contiguous() and row_start.shape[0] == S + 1 and S >= 1, lambda: f"{what}: tables")
+    return S
+
+
+def _history(hist, n_floats, what):
+    """A state tensor [slots, n_floats] whose rows are contiguous; -> a slot's stride in floats."""
+    _dev(hist, "history", (torch.float32,), 2)
+    _need(hist.shape[1] == n_floats and (hist.stride(1) == 1 or n_floats == 1), lambda: f"{what}: history {tuple(hist.shape)}, wanted [slots, {n_floats}]")
+    return hist.stride(0)
+
+
+def rmsnorm(x, weight, eps, out, rows=None):
+    """out[r, :] = x[rows[r], :E] / sqrt(mean(x[.., :E]^2) + eps) * weight, E = out.shape[1] (the first E columns of x;
+    rows None: every row; weight None: no weight).  32-bit statistics; x and out may be the same tensor."""
+    _dev(x, "x", _FLOATS, 2), _dev(out, "out", _FLOATS, 2)
+    E = out.shape[1]
+    ldx, ldo = _rows(x, "x"), _rows(out, "out")
+    _need(x.shape[1] >= E, "rmsnorm: x is narrower than out")
+    _f32vec(weight, "weight", E)
+    if rows is not None:
+        _dev(rows, "rows", _I32, 1)
+        _need(rows.is_contiguous() and rows.shape[0] == out.shape[0], "rmsnorm: rows")
+    else:
+        _need(out.shape[0] == x.shape[0], "rmsnorm: out rows")
+    _ok(_lib("sequence").dn_rmsnorm(x.data_ptr(), _CODE[x.dtype], ldx, _ptr(weight), out.data_ptr(), _CODE[out.dtype], ldo,
+                                    _ptr(rows), out.shape[0], E, float(eps), _stream()), "rmsnorm")
+    return out
+
+
+def concat_cast(a, b, out):
+    """out[t, :] = [a[t, :] | b[t, :]], a and b 32-bit, out contiguous in its own dtype."""
+    _dev(a, "a", (torch.float32,), 2), _dev(b, "b", (torch.float32,), 2), _dev(out, "out", _FLOATS, 2)
+    T = a.shape[0]
+    _need(b.shape[0] == T and tuple(out.shape) == (T, a.shape[1] + b.shape[1]) and out.is_contiguous(), "concat_cast: shapes")
+    _ok(_lib("sequence").dn_concat_cast(a.data_ptr(), _rows(a, "a"), a.shape[1], b.data_ptr(), _rows(b, "b"), b.shape[1],
+                                        out.data_ptr(), _CODE[out.dtype], T, _stream()), "concat_cast")
+    return out
+
+
+def conv_rows(h, w, hist, row_start, slots, out):
+    """out[t, c] = h[t, c] + sum_j w[c, j] h[t - taps + 1 + j, c] inside each request; the rows before a request's first
+    row of this step come from hist [slots, (taps - 1) * width] (oldest first).  h 32-bit [T, width]."""
+    _dev(h, "h", (torch.float32,), 2), _dev(w, "w", (torch.float32,), 2), _dev(out, "out", _FLOATS, 2)
+    T, width = h.shape
+    taps = w.shape[1]
+    S = _request_tables(row_start, slots, "conv_rows")
+    _need(h.is_contiguous() and out.is_contiguous() and w.is_contiguous() and w.shape[0] == width and tuple(out.shape) == (T, width),
+          "conv_rows: shapes")
+    stride = _history(hist, (taps - 1) * width, "conv_rows") if taps > 1 else 0
+    _ok(_lib("sequence").dn_conv_rows(h.data_ptr(), w.data_ptr(), _ptr(hist) if taps > 1 else 0, row_start.data_ptr(),
+                                      slots.data_ptr(), S, T, width, taps, out.data_ptr(), _CODE[out.dtype], stride, _stream()),
+        "conv_rows")
+    return out
+
+
+def history_update(h, hist, row_start, slots):
+    """hist [slots, keep * width]: the last `keep` rows of (a request's history ++ its rows of this step) become its history."""
+    _dev(h, "h", _FLOATS, 2)
+    T, width = h.shape
+    S = _request_tables(row_start, slots, "history_update")
+    _dev(hist, "history", (torch.float32,), 2)
+    _need(h.is_contiguous() and hist.shape[1] % width == 0, "history_update: shapes")
+    keep = hist.shape[1] // width
+    stride = _history(hist, keep * width, "history_update")
+    _ok(_lib("sequence").dn_history_update(h.data_ptr(), _CODE[h.dtype], hist.data_ptr(), row_start.data_ptr(), slots.data_ptr(),
+                                           S, width, keep, stride, _stream()), "history_update")
+
+
+def shift_mix(h, hist, mu, row_start, slots, out):
+    """out[m, t, :] = h[t] + (h[t - 1] - h[t]) * mu[m]; the row before a request's first row of the step is hist[slot]."""
+    _dev(h, "h", _FLOATS, 2), _dev(out, "out", _FLOATS, 3)
+    T, width = h.shape
+    n = mu.shape[0]
+    S = _request_tables(row_start, slots, "shift_mix")
+    _f32vec(mu, "mu", n * width)
+    _need(h.is_contiguous() and out.is_contiguous() and tuple(out.shape) == (n, T, width), "shift_mix: shapes")
+    stride = _history(hist, width, "shift_mix")
+    _ok(_lib("sequence").dn_shift_mix(h.data_ptr(), _CODE[h.dtype], hist.data_ptr(), mu.data_ptr(), n, row_start.data_ptr(),
+                                      slots.data_ptr(), S, T, width, out.data_ptr(), _CODE[out.dtype], stride, _stream()), "shift_mix")
+    return out
+
+
+def rotary(src, dst, positions, freq, n_vec, dims, width, src_off=0, src_stride=None, dst_off=0, dst_stride=None):
+    """Vector n (n < n_vec) of row t, `width` wide, starts at column src_off + n * src_stride of src; of its first `dims`
+    entries, 2i and 2i + 1 are turned by positions[t] * freq[i] (32-bit angles), the rest pass; it goes to column
+    dst_off + n * dst_stride of dst (which may be src)."""
+    _dev(src, "src", _FLOATS, 2), _dev(dst, "dst", _FLOATS, 2), _dev(positions, "positions", _I32, 1)
+    T = src.shape[0]
+    src_stride = width if src_stride is None else src_stride
+    dst_stride = width if dst_stride is None else dst_stride
+    _f32vec(freq, "freq", dims // 2)
+    _need(dst.shape[0] == T and positions.is_contiguous() and positions.shape[0] == T, "rotary: rows")
+    _need(dims % 2 == 0 and 0 <= dims <= width and n_vec >= 0, "rotary: dims")
+    if n_vec:
+        _need(src_off >= 0 and src_off + (n_vec - 1) * src_stride + width <= src.shape[1]
+              and dst_off >= 0 and dst_off + (n_vec - 1) * dst_stride + width <= dst.shape[1], "rotary: vectors outside their rows")
+    _ok(_lib("sequence").dn_rotary(src.data_ptr(), _CODE[src.dtype], _rows(src, "src"), src_off, src_stride, dst.data_ptr(),
+                                   _CODE[dst.dtype], _rows(dst, "dst"), dst_off, dst_stride, positions.data_ptr(), freq.data_ptr(),
+                                   T, n_vec, dims, width, _stream()), "rotary")
+    return dst
+
+
+def activate(x, kind, out, bias=None, lower=None):
+    """out = act(x + bias): "silu", "sigmoid", "tanh", "exp_neg_exp" (exp(-exp(z))), "bounded_sigmoid"
+    (lower + (1 - lower) * sigmoid(z)).  x 32-bit; out may be x."""
+    _dev(x, "x", (torch.float32,), 2), _dev(out, "out", _FLOATS, 2)
+    T, n = x.shape
+    _need(tuple(out.shape) == (T, n), "activate: shapes")
+    _f32vec(bias, "bias", n), _f32vec(lower, "lower", n)
+    _ok(_lib("sequence").dn_activate(x.data_ptr(), _rows(x, "x"), _ptr(bias), _ptr(lower), ACTIVATIONS[kind], out.data_ptr(),
+                                     _CODE[out.dtype], _rows(out, "out"), T, n, _stream()), "activate")
+    return out
+
+
+def gated(x, g, kind, out):
+    """out = x * act(g), act "silu", "sigmoid" or "tanh"; g 32-bit."""
+    _dev(x, "x", _FLOATS, 2), _dev(g, "g", (torch.float32,), 2), _dev(out, "out", _FLOATS, 2)
+    T, n = x.shape
+    _need(tuple(g.shape) == (T, n) and tuple(out.shape) == (T, n) and kind in ("silu", "sigmoid", "tanh"), "gated: shapes")
+    _ok(_lib("sequence").dn_gated(x.data_ptr(), _CODE[x.dtype], _rows(x, "x"), g.data_ptr(), _rows(g, "g"), ACTIVATIONS[kind],
+                                  out.data_ptr(), _CODE[out.dtype], _rows(out, "out"), T, n, _stream()), "gated")
+    return out
+
+
+def state_scan(r, k, v, w, u, state, row_start, slots, n_heads, dk, dv, out, read_after=False, key_from_decay=False):
+    """The recurrence of a matrix state per head, S [dk, dv], over each request's rows of this step in order:
+      a = 1 - w if key_from_decay else k
+      read_after:  S <- diag(w) S + a v^T ;  o = S^T r
+      else:        o = (S + diag(u) a v^T)^T r ;  S <- diag(w) S + a v^T        (u None: no bonus)
+    r, k, w: 32-bit [T, heads * dk]; v, out: 32-bit [T, heads * dv]; state: 32-bit [slots, heads * dk * dv], read and
+    written at the requests' slots."""
+    for t, name, n in ((r, "r", dk), (w, "w", dk), (v, "v", dv), (out, "out", dv)) + (() if key_from_decay else ((k, "k", dk),)):
+        _dev(t, name, (torch.float32,), 2)
+        _need(t.shape[1] == n_heads * n, lambda: f"state_scan: {name} {tuple(t.shape)}")
+    T = r.shape[0]
+    S = _request_tables(row_start, slots, "state_scan")
+    _need(all(t.shape[0] == T for t in (v, w, out)), "state_scan: rows")
+    _need(1 <= dk <= 256, lambda: f"state_scan: {dk} key channels a head; the kernel keeps up to 256 in registers")
+    _f32vec(u, "u", n_heads * dk)
+    stride = _history(state, n_heads * dk * dv, "state_scan")
+    _ok(_lib("sequence").dn_state_scan(r.data_ptr(), _rows(r, "r"), 0 if key_from_decay else k.data_ptr(),
+                                       0 if key_from_decay else _rows(k, "k"), v.data_ptr(), _rows(v, "v"), w.data_ptr(),
+                                       _rows(w, "w"), _ptr(u), state.data_ptr(), stride, row_start.data_ptr(), slots.data_ptr(), S,
+                                       n_heads, dk, dv, int(read_after), int(key_from_decay), out.data_ptr(), _rows(out, "out"),
+                                       _stream()), "state_scan")
+    return out
+
+
+def head_norm(o, weight, eps, out, n_heads, gate=None, gate_kind="silu"):
+    """out[t, h, :] = o[t, h, :] / sqrt(mean(o[t, h, :]^2) + eps) * weight * act(gate[t, h, :]).  weight: None, one per
+    column of o, or one per column of a head (shared by the heads); o and gate 32-bit."""
+    _dev(o, "o", (torch.float32,), 2), _dev(out, "out", _FLOATS, 2)
+    T, n = o.shape
+    _need(n % n_heads == 0 and tuple(out.shape) == (T, n), "head_norm: shapes")
+    dv = n // n_heads
+    w_stride = 0
+    if weight is not None:
+        _f32vec(weight, "weight")
+        _need(weight.numel() in (n, dv), "head_norm: weight")
+        w_stride = dv if weight.numel() == n and n_heads > 1 else 0
+    if gate is not None:
+        _dev(gate, "gate", (torch.float32,), 2)
+        _need(tuple(gate.shape) == (T, n) and gate_kind in ("silu", "sigmoid", "tanh"), "head_norm: gate")
+    _ok(_lib("sequence").dn_head_norm(o.data_ptr(), _rows(o, "o"), _ptr(weight), w_stride, float(eps), _ptr(gate),
+                                      _rows(gate, "gate") if gate is not None else 0, ACTIVATIONS[gate_kind], out.data_ptr(),
+                                      _CODE[out.dtype], _rows(out, "out"), T, n_heads, dv, _stream()), "head_norm")
+    return out
+
+
+# -- a matrix per head, a matrix per expert (csrc/kernels/grouped.hip) -----------------------------------------------------
+def heads_linear(a, w, out, a_off=0, a_stride=None, o_off=0, o_stride=None):
+    """out[t, o_off + h * o_stride + n] = sum_k w[h, n, k] * a[t, a_off + h * a_stride + k]; w [heads, N, K]; 32-bit sums."""
+    _dev(a, "a", _FLOATS, 2), _dev(w, "w", _FLOATS, 3), _dev(out, "out", _FLOATS, 2)
+    H, N, K = w.shape
+    T = a.shape[0]
+    a_stride = K if a_stride is None else a_stride
+    o_stride = N if o_stride is None else o_stride
+    _need(w.is_contiguous() and out.shape[0] == T, "heads_linear: shapes")
+    _need(a_off >= 0 and a_off + (H - 1) * a_stride + K <= a.shape[1] and o_off >= 0 and o_off + (H - 1) * o_stride + N <= out.shape[1],
+          "heads_linear: heads outside their rows")
+    _ok(_lib("grouped").dn_heads_linear(a.data_ptr(), _CODE[a.dtype], _rows(a, "a"), a_off, a_stride, w.data_ptr(), _CODE[w.dtype],
+                                        out.data_ptr(), _CODE[out.dtype], _rows(out, "out"), o_off, o_stride, T, H, N, K, _stream()),
+        "heads_linear")
+    return out
+
+
+def moe_route(z, correction, top, ids, wts):
+    """Per row: s = softmax(z); the `top` experts with the largest s + correction (the lower index wins a tie) go to ids
+    [T, top], their s divided by the sum of the chosen s (+ 1e-20) to wts [T, top]."""
+    _dev(z, "z", (torch.float32,), 2), _dev(ids, "ids", _I32, 2), _dev(wts, "wts", (torch.float32,), 2)
+    T, E = z.shape
+    _need(z.is_contiguous() and ids.is_contiguous() and wts.is_contiguous() and tuple(ids.shape) == (T, top)
+          and tuple(wts.shape) == (T, top) and 1 <= top <= E, "moe_route: shapes")
+    _f32vec(correction, "correction", E)
+    _ok(_lib("grouped").dn_moe_route(z.data_ptr(), _ptr(correction), T, E, top, ids.data_ptr(), wts.data_ptr(), _stream()), "moe_route")
+
+
+def moe_plan(ids, n_experts, offsets, order):
+    """The pairs (row, choice), pair i = row * top + choice, sorted by expert and then by i: order [T * top]; expert e has
+    the places offsets[e] .. offsets[e + 1] - 1 (offsets [experts + 1])."""
+    _dev(ids, "ids", _I32, 2), _dev(offsets, "offsets", _I32, 1), _dev(order, "order", _I32, 1)
+    n = ids.numel()
+    _need(ids.is_contiguous() and offsets.shape[0] == n_experts + 1 and order.shape[0] == n and offsets.is_contiguous()
+          and order.is_contiguous(), "moe_plan: shapes")
+    _ok(_lib("grouped").dn_moe_plan(ids.data_ptr(), n, n_experts, offsets.data_ptr(), order.data_ptr(), _stream()), "moe_plan")
+
+
+def moe_up(h, order, offsets, top, w_gate, w_up, limit, alpha, y):
+    """For place p of expert e, the row t = order[p] // top: g = min(w_gate[e] h[t], limit), u = clamp(w_up[e] h[t], -limit,
+    limit), y[p] = g * sigmoid(alpha * g) * (u + 1).  w_gate, w_up: [experts, ff, width]; y [T * top, ff]."""
+    _dev(h, "h", _FLOATS, 2), _dev(w_gate, "w_gate", _FLOATS, 3), _dev(w_up, "w_up", (w_gate.dtype,), 3), _dev(y, "y", _FLOATS, 2)
+    E, ff, width = w_gate.shape
+    n = order.shape[0]
+    _need(w_gate.is_contiguous() and w_up.is_contiguous() and tuple(w_up.shape) == (E, ff, width) and h.shape[1] == width
+          and y.is_contiguous() and tuple(y.shape) == (n, ff) and offsets.shape[0] == E + 1 and n == h.shape[0] * top, "moe_up: shapes")
+    _ok(_lib("grouped").dn_moe_up(h.data_ptr(), _CODE[h.dtype], _rows(h, "h"), order.data_ptr(), offsets.data_ptr(), E, top, n,
+                                  w_gate.data_ptr(), w_up.data_ptr(), _CODE[w_gate.dtype], ff, width, float(limit), float(alpha),
+                                  y.data_ptr(), _CODE[y.dtype], _stream()), "moe_up")
+
+
+def moe_down(y, order, offsets, w_down, out):
+    """out[order[p], :] = w_down[e] y[p, :] for the places p of expert e; w_down [experts, width, ff]; out 32-bit [T * top, width]."""
+    _dev(y, "y", _FLOATS, 2), _dev(w_down, "w_down", _FLOATS, 3), _dev(out, "out", (torch.float32,), 2)
+    E, width, ff = w_down.shape
+    n = order.shape[0]
+    _need(w_down.is_contiguous() and y.is_contiguous() and tuple(y.shape) == (n, ff) and out.is_contiguous()
+          and tuple(out.shape) == (n, width) and offsets.shape[0] == E + 1, "moe_down: shapes")
+    _ok(_lib("grouped").dn_moe_down(y.data_ptr(), _CODE[y.dtype], order.data_ptr(), offsets.data_ptr(), E, n, w_down.data_ptr(),
+                                    _CODE[w_down.dtype], width, ff, out.data_ptr(), _stream()), "moe_down")
+
+
+def moe_combine(out, wts, x):
+    """x[t, :] += sum_c wts[t, c] * out[t * top + c, :], the choices in their order."""
+    _dev(out, "out", (torch.float32,), 2), _dev(wts, "wts", (torch.float32,), 2), _dev(x, "x", (torch.float32,), 2)
+    T, top = wts.shape
+    width = x.shape[1]
+    _need(out.is_contiguous() and wts.is_contiguous() and tuple(out.shape) == (T * top, width) and x.shape[0] == T, "moe_combine: shapes")
+    _ok(_lib("grouped").dn_moe_combine(out.data_ptr(), wts.data_ptr(), T, top, width, x.data_ptr(), _rows(x, "x"), _stream()),
+        "moe_combine")

@@ -10,6 +10,7 @@ Kinds of part and their registries:
   mixer            MIXERS          forward(h, ctx, cache, accumulate_into) ; cache_spec()
   feed-forward     FEED_FORWARDS   forward(h, ctx, accumulate_into)
   norm             NORMS           forward(x, out_dtype, rows=None) -> tensor
+  input filter     FILTERS         forward(h, ctx, cache) -> what the mixer reads ; cache_spec()
   position code    POSITIONS       table() for the embedding stage, rotate(q, k, ctx) for mixers
   arrangement      ARRANGEMENTS    SLOTS names its parts and their kinds; forward(x, ctx, caches, runtime): how
                                    norms, mixers and feed-forwards stand in a block
@@ -83,6 +84,7 @@ class Part:
     requests on the host, no size taken from a table's contents), so a decode step with it can be
     captured once as a HIP graph and replayed over new tables."""
     graph_safe = False
+    libraries = ()     # kernel libraries (names in build.LIBRARIES) beyond the ones every model needs
 
     def param_specs(self) -> List[ParamSpec]:
         return []
@@ -194,5 +196,6 @@ FEED_FORWARDS = Registry("feed-forward")
 NORMS = Registry("norm")
 POSITIONS = Registry("position encoding")
 ARRANGEMENTS = Registry("block arrangement")
+FILTERS = Registry("input filter")
 # the kinds that an arrangement's SLOTS may name
-KINDS = {"mixer": MIXERS, "feed_forward": FEED_FORWARDS, "norm": NORMS}
+KINDS = {"mixer": MIXERS, "feed_forward": FEED_FORWARDS, "norm": NORMS, "filter": FILTERS}

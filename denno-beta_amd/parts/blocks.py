@@ -88,3 +88,30 @@ class PreNormBlock:
         if stream is not None:
             return LazyNorm(norm, x, runtime.act_dtype, stream)
         return norm.forward(x, runtime.act_dtype, packed=part.packed_input(x.shape[0]))
+
+
+@ARRANGEMENTS.register("pre_norm_filtered")
+class FilteredPreNormBlock:
+    """x += mixer(filter(norm1(x))); x += ffn(norm2(x)).  The filter (a short convolution over time, or none) reads the
+    normed rows in 32-bit and keeps a state of its own, so a call of this block names two caches: the filter's and the
+    mixer's.  A block whose feed-forward is "none" ends after the mixer."""
+
+    SLOTS = {"norm1": "norm", "filter": "filter", "mixer": "mixer", "norm2": "norm", "ffn": "feed_forward"}
+
+    def __init__(self, norm1, filter, mixer, norm2, ffn):
+        self.norm1, self.filter, self.mixer, self.norm2, self.ffn = norm1, filter, mixer, norm2, ffn
+        self.has_ffn = not getattr(ffn, "absent", False)
+
+    def parts(self):
+        return [self.norm1, self.filter, self.mixer] + ([self.norm2, self.ffn] if self.has_ffn else [])
+
+    def mixers(self):
+        return [self.filter, self.mixer]
+
+    def forward(self, x, ctx, caches, runtime):
+        runtime.stream_stats = None
+        h = self.norm1.forward(x, getattr(self.filter, "in_dtype", runtime.act_dtype))
+        h = self.filter.forward(h, ctx, caches[0])
+        self.mixer.forward(h, ctx, caches[1], accumulate_into=x)
+        if self.has_ffn:
+            self.ffn.forward(self.norm2.forward(x, runtime.act_dtype), ctx, accumulate_into=x)

@@ -4,6 +4,7 @@ from __future__ import annotations
 import torch
 
 from ..kernels import ops
+from ..weights.spec import ParamSpec
 from .base import MIXERS, POSITIONS, PagedKV, Part
 from .linear import Linear
 
@@ -98,3 +99,80 @@ class CausalSelfAttention(Part):
                       self.scale, self.window, tiles_wide=g.tiles_wide, single_rows=g.single_rows,
                       max_context=g.max_context)
         self.out(o, residual=accumulate_into, stats=stats, deferred=deferred)
+
+
+@MIXERS.register("latent_attention")
+class LatentAttention(Part):
+    """Causal softmax attention whose keys and values are made from one small vector per token.
+
+    Per token: q = W_q h, per head [dim plain | rot_dim turned]; W_dkv h gives kv_rank numbers, normed without a mean to
+    the latent c, and rot_dim numbers that, turned by the position, are a key part shared by all heads.  Head h's plain
+    key is W_uk[h] c, its value W_uv[h] c; the score is (q_plain . k_plain + q_turned . k_turned) * scale.  The heads'
+    results, times sigmoid(W_g h), go through the output projection.
+
+    Only c and the turned key part are kept, as one key of kv_rank + rot_dim numbers per token that every head reads:
+    q_plain . (W_uk c) = (W_uk^T q_plain) . c, so the query is carried to the latent's space once per token, the
+    attention kernels run with one key head of that width (the same rows serve as values), and W_uv is applied to
+    the weighted sum of latents.  position: the arguments of a "rotary_pairs" encoding for the turned parts."""
+    libraries = ("sequence", "grouped")
+
+    def __init__(self, width: int, n_heads: int, head_dim: int, rot_dim: int, value_dim: int, kv_rank: int, scale: float,
+                 eps: float, position: dict, names: dict):
+        """names: q, dkv, g, uk, uv, o (matrices); dkv_norm (vector)."""
+        self.width, self.n_heads, self.head_dim, self.rot_dim = width, n_heads, head_dim, rot_dim
+        self.value_dim, self.kv_rank, self.scale, self.eps, self.names = value_dim, kv_rank, float(scale), eps, dict(names)
+        self.key_dim = kv_rank + rot_dim
+        if not 1 <= self.key_dim <= 256:
+            raise ValueError(f"latent_attention: a kept key of {self.key_dim} numbers; the attention kernels take up to 256")
+        self.q_width = n_heads * (head_dim + rot_dim)
+        self.o_width = n_heads * value_dim
+        # one product for everything that reads h: q | dkv | g
+        self.proj = Linear(width, self.q_width + self.key_dim + self.o_width, names["q"] + "+dkv+g", None,
+                           weight_sources=((names["q"], self.q_width), (names["dkv"], self.key_dim), (names["g"], self.o_width)))
+        self.out = Linear(self.o_width, width, names["o"], None)
+        self.position = POSITIONS.make(("rotary_pairs", dict(position, head_dim=rot_dim)))
+
+    def param_specs(self):
+        H, r = self.n_heads, self.kv_rank
+        return self.proj.param_specs() + self.out.param_specs() + [
+            ParamSpec(self.names["uk"], (H * self.head_dim, r), "matrix", ("normal", 0.0, r ** -0.5)),
+            ParamSpec(self.names["uv"], (H * self.value_dim, r), "matrix", ("normal", 0.0, r ** -0.5)),
+            ParamSpec(self.names["dkv_norm"], (r,), "vector", ("normal", 1.0, 0.1))]
+
+    def cache_spec(self):
+        return PagedKV(1, self.key_dim)
+
+    def bind(self, tensors, runtime):
+        super().bind(tensors, runtime)
+        self.proj.bind(tensors), self.out.bind(tensors)
+        self.position.bind(tensors, runtime)
+        H, r = self.n_heads, self.kv_rank
+        # W_uk per head, transposed once: [heads, kv_rank, dim], so that both per-head products are out = W[h] a
+        self.uk_t = tensors[self.names["uk"]].view(H, self.head_dim, r).transpose(1, 2).contiguous()
+        self.uv = tensors[self.names["uv"]].view(H, self.value_dim, r).contiguous()
+        self.c_norm = tensors[self.names["dkv_norm"]]
+
+    def forward(self, h, ctx, cache, accumulate_into):
+        act, T, H = self.runtime.act_dtype, h.shape[0], self.n_heads
+        dn, dr, r, kd = self.head_dim, self.rot_dim, self.kv_rank, self.key_dim
+        g = ctx.groups[cache.group]
+        z = self.proj(h, out_dtype=torch.float32)
+        low, gate = self.q_width, self.q_width + kd
+        # the token's key: [c | turned part]
+        key = torch.empty((T, kd), dtype=act, device=h.device)
+        ops.rmsnorm(z[:, low:low + r], self.c_norm, self.eps, key[:, :r])
+        self.position.turn(z, key, ctx.positions, 1, dr, src_off=low + r, dst_off=r)
+        if cache.writes:
+            ops.kv_write(key, 0, 0, g.slot_map, cache.k, cache.v)
+        # the queries in the latent's space: [W_uk^T q_plain | turned part] per head
+        q = torch.empty((T, H * kd), dtype=act, device=h.device)
+        ops.heads_linear(z, self.uk_t, q, a_off=0, a_stride=dn + dr, o_off=0, o_stride=kd)
+        self.position.turn(z, q, ctx.positions, H, dr, src_off=dn, src_stride=dn + dr, dst_off=r, dst_stride=kd)
+        o_lat = torch.empty((T, H * kd), dtype=act, device=h.device)
+        ops.attention(q, o_lat, cache.k, cache.v, g.block_tables, g.tiles, H, self.scale, 0, tiles_wide=g.tiles_wide,
+                      single_rows=g.single_rows, max_context=g.max_context)
+        o = torch.empty((T, self.o_width), dtype=torch.float32, device=h.device)
+        ops.heads_linear(o_lat, self.uv, o, a_off=0, a_stride=kd)
+        og = torch.empty((T, self.o_width), dtype=act, device=h.device)
+        ops.gated(o, z[:, gate:], "sigmoid", og)
+        self.out(og, residual=accumulate_into)

@@ -36,6 +36,7 @@ class LayerCall:
     layer: int                    # index into DecoderSpec.layers
     cache: Union[int, Tuple[int, ...]]   # the cache this call uses; a tuple: one for each mixer of the layer
     writes_cache: bool = True     # False: it only reads what another call wrote
+    inject: Optional[str] = None  # a name in DecoderSpec.injections: done to the stream right before this call
 
     def caches(self) -> Tuple[int, ...]:
         return (self.cache,) if isinstance(self.cache, int) else tuple(self.cache)
@@ -67,6 +68,10 @@ class DecoderSpec:
     logit_softcap: float = 0.0            # > 0: then cap * tanh(logit / cap)
     embedding_scale: float = 1.0          # the token table's rows times this, before the position table's
     extra_embeddings: List[EmbeddingTable] = field(default_factory=list)   # added behind them, in this order
+    embedding_norm: Optional[PartSpec] = None   # a norm of the embedded rows, before the first layer
+    # name -> checkpoint name of a matrix [width, 2 width]: where a LayerCall names it, the stream becomes
+    # W [x ; x0], x the stream as it stands and x0 the embedding stage's output (a loop's way back in)
+    injections: Dict[str, str] = field(default_factory=dict)
     eos_token_ids: Tuple[int, ...] = ()
     # how checkpoints of this architecture name things
     name_prefixes: Tuple[str, ...] = ("",)
@@ -111,6 +116,8 @@ class DecoderModel:
                                  f"the description gives {sorted(ls.parts)}")
             self.blocks.append(cls(**{slot: KINDS[kind].make(ls.parts[slot]) for slot, kind in cls.SLOTS.items()}))
         self.final_norm = NORMS.make(spec.final_norm)
+        self.embedding_norm = NORMS.make(spec.embedding_norm) if spec.embedding_norm is not None else None
+        self.injections = {name: Linear(2 * spec.width, spec.width, weight, None) for name, weight in spec.injections.items()}
         # the head: a matrix of its own, or the token table, transposed
         self.head = Linear(spec.width, spec.vocab, spec.head_weight or spec.token_table, spec.head_bias)
         self._check_run_order()
@@ -127,6 +134,8 @@ class DecoderModel:
         for i, c in enumerate(spec.run_order):
             if not 0 <= c.layer < len(spec.layers):
                 raise ValueError(f"run_order[{i}] names layer {c.layer}; there are {len(spec.layers)}")
+            if c.inject is not None and c.inject not in spec.injections:
+                raise ValueError(f"run_order[{i}] names the injection {c.inject!r}; known: {sorted(spec.injections)}")
             mixers = self.blocks[c.layer].mixers()
             if len(c.caches()) != len(mixers):
                 raise ValueError(f"run_order[{i}] names {len(c.caches())} caches; layer {c.layer} has {len(mixers)} mixers")
@@ -153,6 +162,8 @@ class DecoderModel:
         for b in self.blocks:
             parts += b.parts()
         parts.append(self.final_norm)
+        if self.embedding_norm is not None:
+            parts.append(self.embedding_norm)
         return parts
 
     def param_specs(self) -> List[ParamSpec]:
@@ -168,6 +179,8 @@ class DecoderModel:
                 raise ValueError(f"two parts claim the tensor {t.name!r}")
             seen.add(t.name)
             specs.append(ParamSpec(t.name, (t.rows, self.spec.width), "table", ("normal", 0.0, 0.02)))
+        for lin in self.injections.values():
+            specs += lin.param_specs()
         specs += [s for s in self.head.param_specs() if s.name not in seen]     # (a tied head's weight is the table's)
         return specs
 
@@ -178,6 +191,8 @@ class DecoderModel:
         for p in self.all_parts():
             p.bind(tensors, runtime)
         self.head.bind(tensors)
+        for lin in self.injections.values():
+            lin.bind(tensors)
         self.extra_tables = {t.name: tensors[t.name] for t in self.spec.extra_embeddings}
         for b in self.blocks:
             after = getattr(b, "after_bind", None)     # an arrangement may make its parts ready for each other
@@ -220,8 +235,17 @@ class DecoderModel:
             parts += [(self.extra_tables[t.name], getattr(ctx, t.index), t.scale) for t in self.spec.extra_embeddings]
             ops.embed_sum(parts, x)
         rt.stream_stats = rt.stream_deferred = None      # nobody has left anything for a norm of these rows yet
+        if self.embedding_norm is not None:
+            x = self.embedding_norm.forward(x, torch.float32)
+        x0 = x.clone() if self.injections else None      # (the blocks add into x in place)
         order = self.spec.run_order
         for i, call in enumerate(order):
+            if call.inject is not None:
+                if rt.stream_deferred is not None:
+                    rt.stream_deferred.flush(x)
+                rt.stream_stats = rt.stream_deferred = None
+                both = ops.concat_cast(x, x0, torch.empty((ctx.T, 2 * self.spec.width), dtype=rt.act_dtype, device=rt.device))
+                x = self.injections[call.inject](both, out_dtype=torch.float32)
             nxt = self.blocks[order[i + 1].layer] if i + 1 < len(order) else None
             rt.next_norm = nxt.first_norm() if nxt is not None and hasattr(nxt, "first_norm") else None
             rt.next_takes_deferred = nxt is not None and getattr(nxt, "takes_deferred", False)

@@ -48,3 +48,26 @@ class LayerNorm(Part):
                 return ops.layernorm_join(x, part, bias, self.weight, self.bias, self.eps, out)
             deferred.flush(x)
         return ops.layernorm(x, self.weight, self.bias, self.eps, out, rows)
+
+
+@NORMS.register("rmsnorm")
+class RMSNorm(Part):
+    """x / sqrt(mean(x^2) + eps) * weight, eps inside the root, statistics in 32-bit."""
+    graph_safe = True
+    libraries = ("sequence",)
+
+    def __init__(self, width: int, eps: float, weight_name: str):
+        self.width, self.eps, self.weight_name = width, eps, weight_name
+
+    def param_specs(self):
+        return [ParamSpec(self.weight_name, (self.width,), "vector", ("normal", 1.0, 0.1))]
+
+    def bind(self, tensors, runtime):
+        super().bind(tensors, runtime)
+        self.weight = tensors[self.weight_name]
+
+    def forward(self, x, out_dtype, rows=None, packed=False):
+        # (packed rows are not written here: the consumer's Linear takes a tensor as well)
+        n = x.shape[0] if rows is None else rows.shape[0]
+        out = torch.empty((n, self.width), dtype=out_dtype, device=x.device)
+        return ops.rmsnorm(x, self.weight, self.eps, out, rows)

@@ -8,6 +8,9 @@ not act in a place returns None there / has `rotates = False`.
 """
 from __future__ import annotations
 
+import torch
+
+from ..kernels import ops
 from ..weights.spec import ParamSpec
 from .base import POSITIONS, Part
 
@@ -62,4 +65,38 @@ class NoPositions(Part):
         return None
 
     def rotate(self, q, k, ctx):
+        return q, k
+
+
+@POSITIONS.register("rotary_pairs")
+class RotaryPairs(Part):
+    """Of a vector's first `dims` entries, entry 2i and entry 2i + 1 form a pair (u, v) that the position p turns by
+    the angle p * base^(-2i / dims): (u cos - v sin, v cos + u sin).  The rest of the vector passes.  Angles are
+    32-bit; the frequencies are made once, in 64-bit, and rounded.  head_dim: the width of the vectors that `rotate`
+    finds side by side in q and k; a mixer whose turned parts lie elsewhere calls `turn` with its own layout."""
+    graph_safe = True
+    rotates = True
+    libraries = ("sequence",)
+
+    def __init__(self, dims: int, base: float, head_dim: int = 0):
+        if dims % 2 != 0 or dims < 0:
+            raise ValueError(f"rotary_pairs: {dims} dimensions cannot be paired")
+        self.dims, self.base, self.head_dim = int(dims), float(base), int(head_dim or dims)
+        if self.dims > self.head_dim:
+            raise ValueError(f"rotary_pairs: {dims} dimensions in vectors of {self.head_dim}")
+
+    def bind(self, tensors, runtime):
+        super().bind(tensors, runtime)
+        i = torch.arange(self.dims // 2, dtype=torch.float64)
+        self.freq = (torch.tensor(self.base, dtype=torch.float64) ** (-2.0 * i / max(self.dims, 1))).to(torch.float32).to(runtime.device)
+
+    def table(self):
+        return None
+
+    def turn(self, src, dst, positions, n_vec, width, **layout):
+        return ops.rotary(src, dst, positions, self.freq, n_vec, self.dims, width, **layout)
+
+    def rotate(self, q, k, ctx):
+        for t in (q, k):
+            self.turn(t, t, ctx.positions, t.shape[1] // self.head_dim, self.head_dim)
         return q, k

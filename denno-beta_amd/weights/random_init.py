@@ -36,6 +36,9 @@ def draw(spec: ParamSpec, seed: int, device="cpu") -> torch.Tensor:
         _, mean, std = spec.init
         t = torch.randn(spec.shape, generator=g, dtype=torch.float32, device=device)
         return t * std + mean
+    if kind == "uniform":
+        _, lo, hi = spec.init
+        return torch.rand(spec.shape, generator=g, dtype=torch.float32, device=device) * (hi - lo) + lo
     if kind == "randint":
         _, lo, hi = spec.init
         return torch.randint(lo, hi, spec.shape, generator=g, device=device)

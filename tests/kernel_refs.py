@@ -222,3 +222,183 @@ def linear_qkv(a, w, bias, out, slot_map, k_pool, v_pool, q_width):
     kvw = k_pool.shape[1] * k_pool.shape[3]
     kv_write(out, q_width, q_width + kvw, slot_map, k_pool, v_pool)
     return out[:, :q_width]
+
+
+# -- layers that carry more than keys and values from token to token ---------------------------------------------------
+def _act(kind, z, lower=None):
+    if kind == "silu":
+        return z * torch.sigmoid(z)
+    if kind == "sigmoid":
+        return torch.sigmoid(z)
+    if kind == "tanh":
+        return torch.tanh(z)
+    if kind == "exp_neg_exp":
+        return torch.exp(-torch.exp(z))
+    if kind == "bounded_sigmoid":
+        return lower + (1.0 - lower) * torch.sigmoid(z)
+    raise ValueError(kind)
+
+
+def rmsnorm(x, weight, eps, out, rows=None):
+    E = out.shape[1]
+    src = (x if rows is None else x[rows.long()])[:, :E].float()
+    y = src / torch.sqrt((src * src).mean(dim=-1, keepdim=True) + eps)
+    out.copy_(y if weight is None else y * weight)
+    return out
+
+
+def concat_cast(a, b, out):
+    out.copy_(torch.cat([a, b], dim=1))
+    return out
+
+
+def _requests(row_start, slots):
+    rs, sl = row_start.tolist(), slots.tolist()
+    return [(sl[s], rs[s], rs[s + 1]) for s in range(len(sl)) if sl[s] >= 0]
+
+
+def conv_rows(h, w, hist, row_start, slots, out):
+    width, taps = w.shape
+    res = torch.zeros(h.shape, dtype=torch.float32)
+    for slot, a, b in _requests(row_start, slots):
+        rows = h[a:b] if taps == 1 else torch.cat([hist[slot].view(taps - 1, width), h[a:b]], dim=0)
+        for t in range(b - a):
+            acc = h[a + t].clone()
+            for j in range(taps):
+                acc += w[:, j] * rows[t + j]
+            res[a + t] = acc
+    out.copy_(res)
+    return out
+
+
+def history_update(h, hist, row_start, slots):
+    width = h.shape[1]
+    keep = hist.shape[1] // width
+    for slot, a, b in _requests(row_start, slots):
+        rows = torch.cat([hist[slot].view(keep, width), h[a:b].float()], dim=0)
+        hist[slot] = rows[rows.shape[0] - keep:].reshape(-1)
+
+
+def shift_mix(h, hist, mu, row_start, slots, out):
+    hf = h.float()
+    res = torch.zeros(out.shape, dtype=torch.float32)
+    for slot, a, b in _requests(row_start, slots):
+        prev = torch.cat([hist[slot].view(1, -1), hf[a:b - 1]], dim=0)
+        for m in range(mu.shape[0]):
+            res[m, a:b] = hf[a:b] + (prev - hf[a:b]) * mu[m]
+    out.copy_(res)
+    return out
+
+
+def rotary(src, dst, positions, freq, n_vec, dims, width, src_off=0, src_stride=None, dst_off=0, dst_stride=None):
+    src_stride = width if src_stride is None else src_stride
+    dst_stride = width if dst_stride is None else dst_stride
+    ang = positions.float()[:, None] * freq[None, :]
+    cos, sin = torch.cos(ang), torch.sin(ang)
+    for n in range(n_vec):
+        vec = src[:, src_off + n * src_stride: src_off + n * src_stride + width].float().clone()
+        a, b = vec[:, 0:dims:2].clone(), vec[:, 1:dims:2].clone()
+        vec[:, 0:dims:2] = a * cos - b * sin
+        vec[:, 1:dims:2] = b * cos + a * sin
+        dst[:, dst_off + n * dst_stride: dst_off + n * dst_stride + width] = vec.to(dst.dtype)
+    return dst
+
+
+def activate(x, kind, out, bias=None, lower=None):
+    z = x if bias is None else x + bias
+    out.copy_(_act(kind, z, lower))
+    return out
+
+
+def gated(x, g, kind, out):
+    out.copy_(x.float() * _act(kind, g))
+    return out
+
+
+def state_scan(r, k, v, w, u, state, row_start, slots, n_heads, dk, dv, out, read_after=False, key_from_decay=False):
+    H = n_heads
+    for slot, a, b in _requests(row_start, slots):
+        S = state[slot].view(H, dk, dv).clone()
+        for t in range(a, b):
+            rt, wt, vt = r[t].view(H, dk), w[t].view(H, dk), v[t].view(H, dv)
+            at = (1.0 - wt) if key_from_decay else k[t].view(H, dk)
+            kv = at[:, :, None] * vt[:, None, :]
+            if read_after:
+                S = wt[:, :, None] * S + kv
+                out[t] = torch.einsum("hi,hij->hj", rt, S).reshape(-1)
+            else:
+                bonus = kv * u.view(H, dk)[:, :, None] if u is not None else 0.0
+                out[t] = torch.einsum("hi,hij->hj", rt, S + bonus).reshape(-1)
+                S = wt[:, :, None] * S + kv
+        state[slot] = S.reshape(-1)
+    return out
+
+
+def head_norm(o, weight, eps, out, n_heads, gate=None, gate_kind="silu"):
+    T, n = o.shape
+    dv = n // n_heads
+    y = o.view(T, n_heads, dv)
+    y = y / torch.sqrt((y * y).mean(dim=-1, keepdim=True) + eps)
+    if weight is not None:
+        y = y * (weight.view(n_heads, dv) if weight.numel() == n else weight)
+    y = y.reshape(T, n)
+    if gate is not None:
+        y = y * _act(gate_kind, gate)
+    out.copy_(y)
+    return out
+
+
+def heads_linear(a, w, out, a_off=0, a_stride=None, o_off=0, o_stride=None):
+    H, N, K = w.shape
+    a_stride = K if a_stride is None else a_stride
+    o_stride = N if o_stride is None else o_stride
+    for h in range(H):
+        y = a[:, a_off + h * a_stride: a_off + h * a_stride + K].float() @ w[h].float().t()
+        out[:, o_off + h * o_stride: o_off + h * o_stride + N] = y.to(out.dtype)
+    return out
+
+
+def moe_route(z, correction, top, ids, wts):
+    s = torch.softmax(z, dim=-1)
+    choice = s if correction is None else s + correction
+    for t in range(z.shape[0]):
+        c = choice[t].clone()
+        picked = []
+        for _ in range(top):
+            e = int(torch.argmax(c))           # (the first of equal values)
+            picked.append(e)
+            c[e] = -float("inf")
+        ws = s[t, picked]
+        ids[t] = torch.tensor(picked, dtype=torch.int32)
+        wts[t] = ws / (ws.sum() + 1e-20)
+
+
+def moe_plan(ids, n_experts, offsets, order):
+    flat = ids.reshape(-1).long()
+    idx = torch.sort(flat, stable=True).indices
+    order.copy_(idx.to(torch.int32))
+    counts = torch.bincount(flat, minlength=n_experts)
+    offsets[0] = 0
+    offsets[1:] = torch.cumsum(counts, 0).to(torch.int32)
+
+
+def moe_up(h, order, offsets, top, w_gate, w_up, limit, alpha, y):
+    off = offsets.tolist()
+    for e in range(w_gate.shape[0]):
+        for p in range(off[e], off[e + 1]):
+            x = h[int(order[p]) // top].float()
+            g = torch.clamp(w_gate[e].float() @ x, max=limit)
+            u = torch.clamp(w_up[e].float() @ x, min=-limit, max=limit)
+            y[p] = (g * torch.sigmoid(alpha * g) * (u + 1.0)).to(y.dtype)
+
+
+def moe_down(y, order, offsets, w_down, out):
+    off = offsets.tolist()
+    for e in range(w_down.shape[0]):
+        for p in range(off[e], off[e + 1]):
+            out[int(order[p])] = w_down[e].float() @ y[p].float()
+
+
+def moe_combine(out, wts, x):
+    T, top = wts.shape
+    x += (out.view(T, top, -1) * wts[:, :, None]).sum(dim=1)
