@@ -186,7 +186,9 @@ def forward(cfg, weights, tokens, dtype=torch.float32, keep_layers=False):
             return w[f"l{i}.{name}"]
         if first:
             x = torch.cat([x, x0], dim=-1) @ w["loop.in"].T
-        h = short_conv(rms_norm(x, p("norm1"), eps), p("canon1"))
+        h = rms_norm(x, p("norm1"), eps)
+        if cfg.get("canon"):
+            h = short_conv(h, p("canon1"))
         x = x + MIXERS[layer["type"]](h, p, layer["mixer"], eps)
         if layer.get("mlp"):
             x = x + routed_experts(rms_norm(x, p("norm2"), eps), p, layer["mlp"])

@@ -1,0 +1,185 @@
+"""The kernels of csrc/kernels/sequence.hip and grouped.hip, each alone against its plain reference in
+tests/kernel_refs.py, at sizes that are multiples of nothing, in both precisions of what they read and write."""
+import pytest
+import torch
+
+import kernel_refs as ref
+from denno_beta_amd.kernels import ops
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+DT = [torch.float32, torch.bfloat16]
+
+
+def close(got, want, dtype=torch.float32, what=""):
+    got, want = got.float().cpu(), want.float().cpu()
+    tol = 2e-5 if dtype == torch.float32 else 1.2e-2
+    bound = tol * (1.0 + want.abs())
+    assert bool(((got - want).abs() <= bound).all()), f"{what}: worst {(got - want).abs().max().item():.3g}"
+
+
+def tables(lengths, slots):
+    starts = [0]
+    for n in lengths:
+        starts.append(starts[-1] + n)
+    return (torch.tensor(starts, dtype=torch.int32, device=DEV), torch.tensor(slots, dtype=torch.int32, device=DEV), starts[-1])
+
+
+def both(fn_name, make, outs, dtype=torch.float32):
+    """Runs ops.<fn> on the device and kernel_refs.<fn> on copies on the host; compares the tensors named in `outs`."""
+    args = make()
+    host = [a.detach().cpu().clone() if isinstance(a, torch.Tensor) else a for a in args]
+    getattr(ops, fn_name)(*args)
+    getattr(ref, fn_name)(*host)
+    torch.cuda.synchronize()
+    for i in outs:
+        close(args[i], host[i], dtype, f"{fn_name} argument {i}")
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("width", [7, 96, 1000])
+def test_rmsnorm(dtype, width):
+    x = torch.randn(13, width + 5, device=DEV) * 3
+    w = torch.randn(width, device=DEV)
+    rows = torch.tensor([12, 0, 5], dtype=torch.int32, device=DEV)
+    both("rmsnorm", lambda: (x, w, 1e-5, torch.empty(13, width, dtype=dtype, device=DEV)), [3], dtype)
+    both("rmsnorm", lambda: (x, None, 1e-3, torch.empty(3, width, dtype=dtype, device=DEV), rows), [3], dtype)
+    # in place, 32-bit
+    y = x[:, :width].contiguous()
+    want = ref.rmsnorm(y.cpu(), w.cpu(), 1e-5, torch.empty(13, width))
+    ops.rmsnorm(y, w, 1e-5, y)
+    close(y, want)
+
+
+@pytest.mark.parametrize("taps", [1, 2, 3, 5])
+@pytest.mark.parametrize("dtype", DT)
+def test_conv_rows_and_history(taps, dtype):
+    width = 37
+    row_start, slots, T = tables([1, 7, 2, 3], [2, 0, -1, 3])
+    h = torch.randn(T, width, device=DEV)
+    w = torch.randn(width, taps, device=DEV)
+    hist = torch.randn(5, max(taps - 1, 1) * width, device=DEV)[:, :(taps - 1) * width]
+    both("conv_rows", lambda: (h, w, hist, row_start, slots, torch.zeros(T, width, dtype=dtype, device=DEV)), [5], dtype)
+    if taps > 1:
+        both("history_update", lambda: (h.to(dtype), hist.clone(), row_start, slots), [1])
+
+
+@pytest.mark.parametrize("dtype", DT)
+def test_shift_mix(dtype):
+    width = 50
+    row_start, slots, T = tables([4, 1, 1, 9], [1, 3, 0, -1])
+    h = torch.randn(T, width, device=DEV).to(dtype)
+    state = torch.randn(4, 100 + width, device=DEV)
+    mu = torch.rand(5, width, device=DEV)
+    both("shift_mix", lambda: (h, state[:, 100:], mu, row_start, slots, torch.zeros(5, T, width, dtype=dtype, device=DEV)), [5], dtype)
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("dims,width", [(8, 8), (6, 10), (0, 4), (64, 64)])
+def test_rotary(dtype, dims, width):
+    T, n_vec = 9, 3
+    src = torch.randn(T, 5 + n_vec * (width + 2), device=DEV)
+    pos = torch.tensor([0, 1, 2, 500, 17, 4095, 33, 100000, 7], dtype=torch.int32, device=DEV)
+    freq = (10000.0 ** (-2.0 * torch.arange(dims // 2, dtype=torch.float64) / max(dims, 1))).float().to(DEV)
+    both("rotary", lambda: (src, torch.zeros(T, 3 + n_vec * (width + 7), dtype=dtype, device=DEV), pos, freq, n_vec, dims, width,
+                             5, width + 2, 3, width + 7), [1], dtype)
+
+
+@pytest.mark.parametrize("kind", sorted(ops.ACTIVATIONS))
+def test_activate_and_gated(kind):
+    x = torch.randn(6, 45, device=DEV) * 2
+    bias, lower = torch.randn(45, device=DEV), torch.rand(45, device=DEV)
+    both("activate", lambda: (x, kind, torch.empty(6, 45, device=DEV), bias, lower), [2])
+    if kind in ("silu", "sigmoid", "tanh"):
+        g = torch.randn(6, 45, device=DEV)
+        both("gated", lambda: (x.bfloat16(), g, kind, torch.empty(6, 45, dtype=torch.bfloat16, device=DEV)), [3], torch.bfloat16)
+
+
+@pytest.mark.parametrize("dk,dv,heads", [(16, 16, 2), (48, 32, 3), (5, 70, 1), (64, 64, 4), (100, 9, 2), (130, 20, 1)])
+@pytest.mark.parametrize("mode", ["bonus", "gate"])
+def test_state_scan(dk, dv, heads, mode):
+    row_start, slots, T = tables([1, 12, 3], [2, -1, 0])
+    r, k = torch.randn(T, heads * dk, device=DEV), torch.randn(T, heads * dk, device=DEV)
+    v = torch.randn(T, heads * dv, device=DEV)
+    w = torch.rand(T, heads * dk, device=DEV) * 0.5 + 0.5
+    u = torch.randn(heads * dk, device=DEV)
+    state = torch.randn(3, heads * dk * dv + 11, device=DEV)
+
+    def make():
+        st = state.clone()
+        out = torch.zeros(T, heads * dv, device=DEV)
+        if mode == "bonus":
+            return (r, k, v, w, u, st[:, :heads * dk * dv], row_start, slots, heads, dk, dv, out, False, False)
+        return (r, None, v, w, None, st[:, :heads * dk * dv], row_start, slots, heads, dk, dv, out, True, True)
+    both("state_scan", make, [5, 11])
+
+
+@pytest.mark.parametrize("dtype", DT)
+def test_head_norm(dtype):
+    T, H, dv = 7, 3, 20
+    o, gate = torch.randn(T, H * dv, device=DEV), torch.randn(T, H * dv, device=DEV)
+    both("head_norm", lambda: (o, torch.randn(H * dv, device=DEV), 1e-5, torch.empty(T, H * dv, dtype=dtype, device=DEV), H, gate, "silu"), [3], dtype)
+    both("head_norm", lambda: (o, torch.randn(dv, device=DEV), 1e-5, torch.empty(T, H * dv, dtype=dtype, device=DEV), H), [3], dtype)
+    both("head_norm", lambda: (o, None, 1e-2, torch.empty(T, H * dv, dtype=dtype, device=DEV), H), [3], dtype)
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("T,H,N,K", [(1, 2, 24, 16), (19, 3, 70, 33), (130, 1, 5, 100)])
+def test_heads_linear(dtype, T, H, N, K):
+    a = torch.randn(T, 4 + H * (K + 3), device=DEV).to(dtype)
+    w = (torch.randn(H, N, K, device=DEV) / K ** 0.5).to(dtype)
+    both("heads_linear", lambda: (a, w, torch.zeros(T, 2 + H * (N + 1), dtype=dtype, device=DEV), 4, K + 3, 2, N + 1), [2], dtype)
+
+
+@pytest.mark.parametrize("T,E,top", [(1, 4, 2), (50, 16, 3), (700, 5, 5), (33, 70, 1)])
+def test_route_and_plan(T, E, top):
+    z = torch.randn(T, E, device=DEV) * 2
+    corr = torch.randn(E, device=DEV) * 0.1
+    ids, wts = torch.zeros(T, top, dtype=torch.int32, device=DEV), torch.zeros(T, top, device=DEV)
+    ops.moe_route(z, corr, top, ids, wts)
+    hi, hw = torch.zeros(T, top, dtype=torch.int32), torch.zeros(T, top)
+    ref.moe_route(z.cpu(), corr.cpu(), top, hi, hw)
+    assert torch.equal(ids.cpu(), hi)
+    close(wts, hw)
+    offsets, order = torch.zeros(E + 1, dtype=torch.int32, device=DEV), torch.zeros(T * top, dtype=torch.int32, device=DEV)
+    ops.moe_plan(ids, E, offsets, order)
+    ho, hr = torch.zeros(E + 1, dtype=torch.int32), torch.zeros(T * top, dtype=torch.int32)
+    ref.moe_plan(hi, E, ho, hr)
+    assert torch.equal(offsets.cpu(), ho) and torch.equal(order.cpu(), hr)
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("T,E,top,ff,width", [(1, 3, 2, 8, 24), (45, 6, 3, 70, 50), (300, 4, 1, 33, 96)])
+def test_experts(dtype, T, E, top, ff, width):
+    h = torch.randn(T, width, device=DEV).to(dtype)
+    wg, wu = ((torch.randn(E, ff, width, device=DEV) / width ** 0.5).to(dtype) for _ in range(2))
+    wd = (torch.randn(E, width, ff, device=DEV) / ff ** 0.5).to(dtype)
+    ids = torch.stack([torch.randperm(E, device=DEV)[:top] for _ in range(T)]).int()
+    offsets, order = torch.zeros(E + 1, dtype=torch.int32, device=DEV), torch.zeros(T * top, dtype=torch.int32, device=DEV)
+    ops.moe_plan(ids, E, offsets, order)
+    y = torch.zeros(T * top, ff, dtype=dtype, device=DEV)
+    ops.moe_up(h, order, offsets, top, wg, wu, 1.5, 1.702, y)
+    hy = torch.zeros(T * top, ff, dtype=dtype)
+    ref.moe_up(h.cpu(), order.cpu(), offsets.cpu(), top, wg.cpu(), wu.cpu(), 1.5, 1.702, hy)
+    close(y, hy, dtype, "moe_up")
+    out = torch.zeros(T * top, width, device=DEV)
+    ops.moe_down(y, order, offsets, wd, out)
+    ho = torch.zeros(T * top, width)
+    ref.moe_down(y.cpu(), order.cpu(), offsets.cpu(), wd.cpu(), ho)
+    close(out, ho, dtype, "moe_down")
+    wts = torch.rand(T, top, device=DEV)
+    x = torch.randn(T, width, device=DEV)
+    hx = x.cpu().clone()
+    ops.moe_combine(out, wts, x)
+    ref.moe_combine(out.cpu(), wts.cpu(), hx)
+    close(x, hx)
+
+
+def test_a_row_does_not_depend_on_its_neighbours():
+    """The same row alone and among others: the same bits from every kernel that works on tiles of rows."""
+    H, N, K = 2, 40, 24
+    a = torch.randn(50, H * K, device=DEV)
+    w = torch.randn(H, N, K, device=DEV)
+    many = ops.heads_linear(a, w, torch.zeros(50, H * N, device=DEV))
+    one = ops.heads_linear(a[17:18].contiguous(), w, torch.zeros(1, H * N, device=DEV))
+    assert torch.equal(many[17:18], one)
