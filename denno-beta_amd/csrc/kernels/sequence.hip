@@ -74,7 +74,10 @@ __global__ __launch_bounds__(256) void conv_rows_kernel(const float* h, const fl
   const int t = blockIdx.x;
   const int s = request_of(row_start, S, t);
   const int slot = slots[s];
-  if (slot < 0) return;
+  if (slot < 0 || t >= row_start[S]) {      // a padding row: zeros, so that what follows works on numbers
+    for (int c = threadIdx.x; c < width; c += 256) store_as(out, static_cast<size_t>(t) * width + c, out_dt, 0.f);
+    return;
+  }
   const int i = t - row_start[s];
   const float* past = hist + static_cast<size_t>(slot) * hist_stride;
   for (int c = threadIdx.x; c < width; c += 256) {
@@ -113,7 +116,11 @@ __global__ __launch_bounds__(256) void shift_mix_kernel(const void* h, int h_dt,
   const int t = blockIdx.x;
   const int s = request_of(row_start, S, t);
   const int slot = slots[s];
-  if (slot < 0) return;
+  if (slot < 0 || t >= row_start[S]) {      // a padding row
+    for (int c = threadIdx.x; c < width; c += 256)
+      for (int m = 0; m < n_mix; ++m) store_as(out, (static_cast<size_t>(m) * T + t) * width + c, out_dt, 0.f);
+    return;
+  }
   const bool first = t == row_start[s];
   for (int c = threadIdx.x; c < width; c += 256) {
     const float cur = load_as(h, static_cast<size_t>(t) * width + c, h_dt);

@@ -330,7 +330,9 @@ class DecodeGraphs:
         slots = mgr.reserve_step(rids, new_lens)
         B = batch_bucket(n, runner.options.max_live)
         # (contexts in buckets of 256, but no bucket beyond what a block table holds: whole pages up to the model's positions)
-        held = min(-(-spec.max_positions // l.page_size) * l.page_size for l in runner.cache.layouts if l.kind == 0)
+        # (a model that keeps no pages at all, only states, has the model's positions for its bound)
+        held = min((-(-spec.max_positions // l.page_size) * l.page_size for l in runner.cache.layouts if l.kind == 0),
+                   default=spec.max_positions)
         ctx_bucket = min(-(-int(new_lens.max()) // DECODE_SPLIT) * DECODE_SPLIT, held)
         key = (B, ctx_bucket)
         g = self.graphs.get(key)

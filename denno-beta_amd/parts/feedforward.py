@@ -76,6 +76,7 @@ class RoutedExperts(Part):
     (+ 1e-20).  An expert: g = min(W_gate h, limit), u = clamp(W_up h, -limit, limit), W_down (g sigmoid(alpha g) (u + 1)).
     The step's (token, expert) pairs are sorted by expert on the device, each expert's products run over tiles of its
     own rows, and the results are added into the stream per token in the order of its choices."""
+    graph_safe = True
     libraries = ("grouped",)
 
     def __init__(self, width: int, inner: int, n_experts: int, top: int, limit: float, alpha: float, router: str,

@@ -27,6 +27,7 @@ class CausalConv(Part):
     """h_t + sum_j w[:, j] h_(t - taps + 1 + j): a convolution over time on every channel, nothing before a request's
     first token.  The last taps - 1 rows it has read are a request's state, so a prompt may come in portions.  It
     reads 32-bit rows and writes the engine's activation dtype."""
+    graph_safe = True
     libraries = ("sequence",)
     in_dtype = torch.float32
 

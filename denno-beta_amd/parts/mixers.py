@@ -114,6 +114,7 @@ class LatentAttention(Part):
     q_plain . (W_uk c) = (W_uk^T q_plain) . c, so the query is carried to the latent's space once per token, the
     attention kernels run with one key head of that width (the same rows serve as values), and W_uv is applied to
     the weighted sum of latents.  position: the arguments of a "rotary_pairs" encoding for the turned parts."""
+    graph_safe = True
     libraries = ("sequence", "grouped")
 
     def __init__(self, width: int, n_heads: int, head_dim: int, rot_dim: int, value_dim: int, kv_rank: int, scale: float,

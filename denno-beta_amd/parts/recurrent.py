@@ -18,6 +18,7 @@ class WKV(Part):
     plain projections, the gate silu(W_g .), the decay w = exp(-exp(W_2 tanh(W_1 .) + w0)) per head and key channel.
     o_t = (S + diag(u) k v^T)^T r, then S <- diag(w) S + k v^T; each head's o is divided by its root mean square,
     times a weight per column, times the gate, then the output projection.  State: S in 32-bit and the last row."""
+    graph_safe = True
     libraries = ("sequence",)
 
     def __init__(self, width: int, n_heads: int, head_dim: int, eps: float, lora: int, names: dict):
@@ -74,6 +75,7 @@ class HGRN2(Part):
     """The forget gate f = lower + (1 - lower) sigmoid(W_f h + b) per head and channel also decides what is written:
     S <- diag(f) S + (1 - f) v^T, o = S^T q with q = silu(W_q h); each head's o is normed over its value columns with
     one weight shared by the heads, then the output projection.  State: S in 32-bit."""
+    graph_safe = True
     libraries = ("sequence",)
 
     def __init__(self, width: int, n_heads: int, head_dim: int, value_dim: int, eps: float, names: dict):
