@@ -15,6 +15,9 @@ decode steps and prefill (`fp32`).  Peaks are the published ones of MI355X.
     python bench.py --only serving [--dtype float32]         BASELINE.json's configs[3] through the scheduler
     python bench.py --only replay [--sequences 8] [--shape xl]   BASELINE.json's configs[4] (or configs[2]'s sizes)
                                                              against the plain implementation, in four ways of cutting
+    python bench.py --only ridopel [--width 1024] [--kernel-times]   four Ridopel layers (latent attention, hgrn2, latent
+                                                             attention, wkv, each with sixteen experts) beside four GPT-2
+                                                             layers of the same width: prefill and decode
 """
 import argparse
 import json
@@ -49,12 +52,17 @@ def baseline_config(index, n_layer=0):
 class Workloads:
     """The decode and prefill measurements on one runner."""
 
-    def __init__(self, a, dtype):
+    def __init__(self, a, dtype, cfg=None):
+        """cfg: a config.json of any architecture with the keys n_positions and vocab_size beside its own (default:
+        the shape that --shape names)."""
         import torch
         from denno_beta_amd.config import EngineOptions
         from denno_beta_amd.engine import ModelRunner
         self.torch, self.a, self.dtype = torch, a, dtype
-        self.cfg, self.full_layers = baseline_config({"xl": 2, "large": 3, "medium": 4}[a.shape], a.layers)
+        if cfg is None:
+            self.cfg, self.full_layers = baseline_config({"xl": 2, "large": 3, "medium": 4}[a.shape], a.layers)
+        else:
+            self.cfg, self.full_layers = cfg, 0
         P = self.cfg["n_positions"]
         live = max(64, a.batch)
         self.opts = EngineOptions(dtype=dtype, page_size=a.page_size, cache_tokens=live * P, max_live=live, max_batch_tokens=4096,
@@ -66,8 +74,9 @@ class Workloads:
     def prompt(self, n):
         return self.torch.randint(0, self.cfg["vocab_size"], (n,), generator=self.gen).tolist()
 
-    def decode(self, batch, steps, warmup, blocks=3):
-        """-> {ms, tok_s, bytes, frac, mean_context}: the median block of `steps` steps."""
+    def decode(self, batch, steps, warmup, blocks=3, on_start=None):
+        """-> {ms, tok_s, bytes, frac, mean_context}: the median block of `steps` steps.  on_start: called once the
+        prompts are in the cache and the warm-up steps are done, before the first timed step."""
         from denno_beta_amd.engine import Engine, SamplingParams
         a, P, sync = self.a, self.cfg["n_positions"], self.torch.cuda.synchronize
         steps = max(1, min(steps, (P - a.context - warmup - 2) // blocks))
@@ -81,6 +90,9 @@ class Workloads:
             eng.step()
         for _ in range(warmup):
             eng.step()
+        if on_start is not None:
+            sync()
+            on_start()
         times = []
         for _ in range(blocks):
             sync()
@@ -119,10 +131,10 @@ class Workloads:
                 runner.end_request(1000 + j)
         t = statistics.median(times[1:])
         cfg = self.cfg
-        V, E = cfg["vocab_size"], cfg["n_embd"]
+        V, E = cfg["vocab_size"], cfg.get("n_embd", cfg.get("width"))
         mat = sum(w.numel() for w in _layer_matrices(runner))
         tokens = 1024 * prompts
-        flops = 2.0 * tokens * mat + 2.0 * prompts * V * E + cfg["n_layer"] * prompts * (4.0 * E * 1024 * 1025 / 2)
+        flops = 2.0 * tokens * mat + 2.0 * prompts * V * E + cfg.get("n_layer", len(cfg.get("layers", ()))) * prompts * (4.0 * E * 1024 * 1025 / 2)
         return {"value": tokens / t, "tokens": tokens, "ms": t * 1e3, "frac": flops / t / MFMA_PEAK[SHORT[self.dtype]]}
 
 
@@ -175,7 +187,8 @@ def main():
     ap.add_argument("--shape", choices=["xl", "large", "medium"], default=None,
                     help="--only decode / prefill / replay: the layer sizes of BASELINE.json's configs[2], [3] or [4] "
                          "(default xl; for replay medium)")
-    ap.add_argument("--only", choices=["decode", "prefill", "serving", "replay"], default=None,
+    ap.add_argument("--width", type=int, default=0, help="--only ridopel: one width instead of 1,024 and 2,048")
+    ap.add_argument("--only", choices=["decode", "prefill", "serving", "replay", "ridopel"], default=None,
                     help="run one workload and print a short line (decode, prefill: for profiling; serving: "
                          "BASELINE.json's configs[3], GPT-2 Large shape, 64 requests through the scheduler; replay: "
                          "configs[4], GPT-2 Medium shape, against the plain implementation)")
@@ -185,6 +198,8 @@ def main():
         sys.exit(2)
     if a.only == "serving":
         return serving(a)
+    if a.only == "ridopel":
+        return ridopel(a)
     if a.only == "replay":
         a.shape = a.shape or "medium"      # (configs[4] as written; --shape xl: the same replay at configs[2]'s sizes)
         return replay(a)
@@ -242,6 +257,55 @@ def main():
             f = Workloads(a, "float32")
             f1, f8 = f.decode(1, min(a.steps, 10), 2), f.decode(8, min(a.steps, 10), 2)
             out["fp32"] = {"decode_b1": keep(f1), "decode_b8": keep(f8), "prefill": f.prefill()}
+    print(json.dumps(out))
+
+
+def ridopel_configs(width, layers=4, vocab=32000, positions=2048):
+    """-> (a Ridopel config, a GPT-2 config) of the same width, layers, vocabulary and positions.  The Ridopel layers
+    take turns between latent attention (heads of 64 + 32, a kept key of 224 + 32 numbers), hgrn2 (heads of 64 keys x 128
+    values) and wkv (heads of 64), each with sixteen experts of the model's width of which a token uses two."""
+    H = width // 128
+    moe = dict(kind="moe", expert=dict(ff=width, limit=7.0), router=dict(experts=16, top=2))
+    lat = dict(type="latent_attention", mlp=moe, mixer=dict(heads=H, dim=64, rot_dim=32, vdim=128, kv_rank=224, scale=96 ** -0.5,
+                                                            rot=dict(base=500000.0, dims=32)))
+    kinds = [lat, dict(type="hgrn2", mlp=moe, mixer=dict(heads=H, dim=64, vdim=128)), lat,
+             dict(type="wkv", mlp=moe, mixer=dict(heads=width // 64, dim=64, decay_rank=64))]
+    rid = dict(architecture="Ridopel", vocab=vocab, width=width, norm=dict(eps=1e-5), canon=dict(taps=4), logit_softcap=30.0,
+               layers=[kinds[i % 4] for i in range(layers)], max_positions=positions, n_positions=positions, vocab_size=vocab)
+    gpt = dict(architectures=["GPT2LMHeadModel"], n_layer=layers, n_embd=width, n_head=width // 64, n_inner=4 * width,
+               vocab_size=vocab, n_positions=positions, layer_norm_epsilon=1e-5, activation_function="gelu_new")
+    return rid, gpt
+
+
+def ridopel(a):
+    """Prefill (two prompts of 1,024 tokens in one step) and decode steps (batch 8 and 64 from a context of 512) of four
+    Ridopel layers beside four GPT-2 layers of the same width; with --kernel-times each model's kernels, launch by launch."""
+    import torch
+    from denno_beta_amd.kernels import ops
+    out = {}
+    for width in ([a.width] if a.width else [1024, 2048]):
+        for name, cfg in zip(("ridopel", "gpt2"), ridopel_configs(width, a.layers or 4)):
+            w = Workloads(a, a.dtype, cfg)
+            rec = {"weight_bytes": w.runner.model.weight_bytes(), "cache_bytes_per_token": w.runner.cache.bytes_per_token()}
+            w.prefill(1, a.prompts)
+            if a.kernel_times:
+                ops.time_launches(True)
+                w.prefill(1, a.prompts)
+                kernel_table(f"{name} width {width}: prefill of {a.prompts} x 1,024 tokens, {a.dtype}")
+                for batch in (8, 64):
+                    w.decode(batch, 4, 1, blocks=1, on_start=lambda: ops.time_launches(True))
+                    kernel_table(f"{name} width {width}: 4 decode steps at batch {batch} from a context of {a.context}, {a.dtype}")
+                    ops.time_launches(False)
+                ops.time_launches(False)
+            else:
+                p = w.prefill(3, a.prompts)
+                rec["prefill_tok_s"], rec["prefill_ms"] = p["value"], p["ms"]
+                for batch in (8, 64):
+                    d = w.decode(batch, min(a.steps, 50), a.warmup)
+                    rec[f"decode_b{batch}_ms"], rec[f"decode_b{batch}_tok_s"] = d["ms"], d["tok_s"]
+            out[f"{name}_{width}"] = rec
+            del w
+            torch.cuda.empty_cache()
     print(json.dumps(out))
 
 

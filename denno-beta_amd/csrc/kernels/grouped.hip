@@ -154,6 +154,43 @@ __global__ __launch_bounds__(256) void plan_kernel(const int* ids, int n, int E,
   }
 }
 
+// The same plan for up to 48 experts, without the walk over each chunk: thread t owns the run of pairs
+// [t L, (t + 1) L), counts them by expert into cnt[t][e] (LDS), thread e then turns column e into each run's first
+// place, and every thread puts its run's pairs there in order.
+__global__ __launch_bounds__(256) void plan_runs_kernel(const int* ids, int n, int E, int* offsets, int* order) {
+  extern __shared__ int cnt[];      // [256][E]
+  const int tid = threadIdx.x;
+  const int L = (n + 255) / 256, lo = min(tid * L, n), hi = min(lo + L, n);
+  for (int e = 0; e < E; ++e) cnt[tid * E + e] = 0;
+  for (int i = lo; i < hi; ++i) cnt[tid * E + ids[i]] += 1;
+  __syncthreads();
+  __shared__ int total[49];
+  if (tid < E) {
+    int run = 0;
+    for (int t = 0; t < 256; ++t) {
+      const int c = cnt[t * E + tid];
+      cnt[t * E + tid] = run;
+      run += c;
+    }
+    total[tid] = run;
+  }
+  __syncthreads();
+  if (tid == 0) {
+    int run = 0;
+    for (int e = 0; e < E; ++e) {
+      offsets[e] = run;
+      run += total[e];
+    }
+    offsets[E] = run;
+    for (int e = 0; e < E; ++e) total[e] = offsets[e];
+  }
+  __syncthreads();
+  for (int i = lo; i < hi; ++i) {
+    const int e = ids[i];
+    order[total[e] + cnt[tid * E + e]++] = i;
+  }
+}
+
 // which expert and which of its tiles of 16 places workgroup `id` has; false: none
 __device__ __forceinline__ bool expert_tile(const int* offsets, int E, int id, int& e, int& p0, int& p1) {
   for (e = 0; e < E; ++e) {
@@ -231,6 +268,159 @@ __global__ __launch_bounds__(256) void combine_kernel(const float* out, const fl
   }
 }
 
+// ---- the same products on the matrix cores (bfloat16) ------------------------------------------------------------
+// A workgroup of four waves takes 64 rows x 64 columns, a wave 32 x 32 as 2 x 2 blocks of v_mfma_f32_16x16x32_bf16.
+// Operands go from memory straight into the lanes that the instruction reads them from: lane l holds the 8 numbers
+// from k = 8 (l / 16) of row (or column) l % 16, 16 bytes in one load, so a step of 32 along K is one load per block
+// and lane, no LDS and no barrier; the waves of a workgroup share their rows and columns through the vector cache.
+// A block's sums: lane l holds row l % 16, columns 4 (l / 16) .. + 3.  Rows beyond a tile's last are read from its
+// last row and stored nowhere.  K is a multiple of 32; every row starts at a multiple of 16 bytes.
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
+constexpr int MT = 64;      // rows of a workgroup's tile
+
+__device__ __forceinline__ bf16x8 load8(const bf16_t* p) { return *reinterpret_cast<const bf16x8*>(p); }
+
+// acc[i][j] += A[rows i] . W[cols j]^T over K; a_ptr[i], w_ptr[j]: this lane's row of block i / column of block j, at
+// its own k offset
+template <bool DUAL>
+__device__ __forceinline__ void mfma_tile(const bf16_t* const a_ptr[2], const bf16_t* const w_ptr[2], const bf16_t* const w2_ptr[2],
+                                          int K, f32x4 acc[2][2], f32x4 acc2[2][2]) {
+#pragma unroll 2
+  for (int k0 = 0; k0 < K; k0 += 32) {
+    bf16x8 af[2], wf[2], wf2[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) af[i] = load8(a_ptr[i] + k0);
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      wf[j] = load8(w_ptr[j] + k0);
+      if (DUAL) wf2[j] = load8(w2_ptr[j] + k0);
+    }
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[j], af[i], acc[i][j], 0, 0, 0);
+        if (DUAL) acc2[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf2[j], af[i], acc2[i][j], 0, 0, 0);
+      }
+  }
+}
+
+// which expert and which of its tiles of 64 places workgroup `id` has
+__device__ __forceinline__ bool expert_tile64(const int* offsets, int E, int id, int& e, int& p0, int& p1) {
+  for (e = 0; e < E; ++e) {
+    const int cnt = offsets[e + 1] - offsets[e];
+    const int tiles = (cnt + MT - 1) / MT;
+    if (id < tiles) {
+      p0 = offsets[e] + id * MT;
+      p1 = min(p0 + MT, offsets[e + 1]);
+      return true;
+    }
+    id -= tiles;
+  }
+  return false;
+}
+
+__global__ __launch_bounds__(256) void expert_up_mfma_kernel(const bf16_t* h, size_t ldh, const int* order, const int* offsets, int E,
+                                                             int top, const bf16_t* wg, const bf16_t* wu, int ff, int width,
+                                                             float limit, float alpha, bf16_t* y) {
+  int e, p0, p1;
+  if (!expert_tile64(offsets, E, blockIdx.x, e, p0, p1)) return;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int pw = p0 + (wave >> 1) * 32, nw = blockIdx.y * 64 + (wave & 1) * 32;
+  if (pw >= p1 || nw >= ff) return;
+  const int kq = (lane >> 4) * 8, lr = lane & 15;
+  const bf16_t *a_ptr[2], *g_ptr[2], *u_ptr[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int p = min(pw + 16 * i + lr, p1 - 1);
+    a_ptr[i] = h + static_cast<size_t>(order[p] / top) * ldh + kq;
+    const size_t n = min(nw + 16 * i + lr, ff - 1);
+    g_ptr[i] = wg + (static_cast<size_t>(e) * ff + n) * width + kq;
+    u_ptr[i] = wu + (static_cast<size_t>(e) * ff + n) * width + kq;
+  }
+  f32x4 g[2][2] = {}, u[2][2] = {};
+  mfma_tile<true>(a_ptr, g_ptr, u_ptr, width, g, u);
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int p = pw + 16 * i + lr;
+    if (p >= p1) continue;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int n = nw + 16 * j + (lane >> 4) * 4;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        if (n + r >= ff) continue;
+        const float gv = fminf(g[i][j][r], limit), uv = fminf(fmaxf(u[i][j][r], -limit), limit);
+        y[static_cast<size_t>(p) * ff + n + r] = from_float<bf16_t>(gv / (1.0f + expf(-alpha * gv)) * (uv + 1.0f));
+      }
+    }
+  }
+}
+
+__global__ __launch_bounds__(256) void expert_down_mfma_kernel(const bf16_t* y, const int* order, const int* offsets, int E,
+                                                               const bf16_t* wd, int width, int ff, float* out) {
+  int e, p0, p1;
+  if (!expert_tile64(offsets, E, blockIdx.x, e, p0, p1)) return;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int pw = p0 + (wave >> 1) * 32, nw = blockIdx.y * 64 + (wave & 1) * 32;
+  if (pw >= p1 || nw >= width) return;
+  const int kq = (lane >> 4) * 8, lr = lane & 15;
+  const bf16_t *a_ptr[2], *w_ptr[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    a_ptr[i] = y + static_cast<size_t>(min(pw + 16 * i + lr, p1 - 1)) * ff + kq;
+    w_ptr[i] = wd + (static_cast<size_t>(e) * width + min(nw + 16 * i + lr, width - 1)) * ff + kq;
+  }
+  f32x4 acc[2][2] = {};
+  mfma_tile<false>(a_ptr, w_ptr, nullptr, ff, acc, nullptr);
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int p = pw + 16 * i + lr;
+    if (p >= p1) continue;
+    const size_t pair = order[p];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int n = nw + 16 * j + (lane >> 4) * 4;
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        if (n + r < width) out[pair * width + n + r] = acc[i][j][r];
+    }
+  }
+}
+
+// out[t, o_off + h * o_stride + n] = sum_k W[h][n][k] a[t, a_off + h * a_stride + k], bfloat16 in, 32-bit sums
+__global__ __launch_bounds__(256) void heads_linear_mfma_kernel(const bf16_t* A, size_t lda, int a_off, int a_stride, const bf16_t* W,
+                                                                void* out, int out_dt, size_t ldo, int o_off, int o_stride, int T,
+                                                                int N, int K) {
+  const int hd = blockIdx.z, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int tw = blockIdx.x * MT + (wave >> 1) * 32, nw = blockIdx.y * 64 + (wave & 1) * 32;
+  if (tw >= T || nw >= N) return;
+  const int kq = (lane >> 4) * 8, lr = lane & 15;
+  const bf16_t *a_ptr[2], *w_ptr[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    a_ptr[i] = A + static_cast<size_t>(min(tw + 16 * i + lr, T - 1)) * lda + a_off + static_cast<size_t>(hd) * a_stride + kq;
+    w_ptr[i] = W + (static_cast<size_t>(hd) * N + min(nw + 16 * i + lr, N - 1)) * K + kq;
+  }
+  f32x4 acc[2][2] = {};
+  mfma_tile<false>(a_ptr, w_ptr, nullptr, K, acc, nullptr);
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int t = tw + 16 * i + lr;
+    if (t >= T) continue;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int n = nw + 16 * j + (lane >> 4) * 4;
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        if (n + r < N) store_as(out, static_cast<size_t>(t) * ldo + o_off + static_cast<size_t>(hd) * o_stride + n + r, out_dt, acc[i][j][r]);
+    }
+  }
+}
+
+bool aligned16(const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; }
+
 bool float_kind(int dt) { return dt == DN_F32 || dt == DN_BF16; }
 
 }  // namespace
@@ -242,6 +432,13 @@ int dn_heads_linear(const void* a, int a_dt, long long lda, int a_off, int a_str
   if (!float_kind(a_dt) || !float_kind(w_dt) || !float_kind(out_dt)) return DN_ERR_DTYPE;
   if (H < 1 || N < 1 || K < 1 || H > 65535) return DN_ERR_SHAPE;
   if (T == 0) return 0;
+  if (a_dt == DN_BF16 && w_dt == DN_BF16 && K % 32 == 0 && lda % 8 == 0 && a_off % 8 == 0 && a_stride % 8 == 0 && aligned16(a) &&
+      aligned16(w)) {
+    hipLaunchKernelGGL(heads_linear_mfma_kernel, dim3((T + MT - 1) / MT, (N + 63) / 64, H), dim3(256), 0, stream,
+                       static_cast<const bf16_t*>(a), static_cast<size_t>(lda), a_off, a_stride, static_cast<const bf16_t*>(w), out,
+                       out_dt, static_cast<size_t>(ldo), o_off, o_stride, T, N, K);
+    return dn_launch_status();
+  }
   hipLaunchKernelGGL(heads_linear_kernel, dim3((T + TM - 1) / TM, (N + TN - 1) / TN, H), dim3(256), 0, stream, a, a_dt,
                      static_cast<size_t>(lda), a_off, a_stride, w, w_dt, out, out_dt, static_cast<size_t>(ldo), o_off, o_stride, T, N, K);
   return dn_launch_status();
@@ -256,7 +453,10 @@ int dn_moe_route(const float* z, const float* correction, int T, int E, int top,
 
 int dn_moe_plan(const int* ids, int n, int E, int* offsets, int* order, hipStream_t stream) {
   if (E < 1 || E > 8192) return DN_ERR_SHAPE;
-  hipLaunchKernelGGL(plan_kernel, dim3(1), dim3(256), (E + 256) * sizeof(int), stream, ids, n, E, offsets, order);
+  if (E <= 48)
+    hipLaunchKernelGGL(plan_runs_kernel, dim3(1), dim3(256), 256 * E * sizeof(int), stream, ids, n, E, offsets, order);
+  else
+    hipLaunchKernelGGL(plan_kernel, dim3(1), dim3(256), (E + 256) * sizeof(int), stream, ids, n, E, offsets, order);
   return dn_launch_status();
 }
 
@@ -264,6 +464,13 @@ int dn_moe_up(const void* h, int h_dt, long long ldh, const int* order, const in
               const void* wu, int w_dt, int ff, int width, float limit, float alpha, void* y, int y_dt, hipStream_t stream) {
   if (!float_kind(h_dt) || !float_kind(w_dt) || !float_kind(y_dt)) return DN_ERR_DTYPE;
   if (n == 0) return 0;
+  if (h_dt == DN_BF16 && w_dt == DN_BF16 && y_dt == DN_BF16 && width % 32 == 0 && ldh % 8 == 0 && aligned16(h) && aligned16(wg) &&
+      aligned16(wu)) {
+    hipLaunchKernelGGL(expert_up_mfma_kernel, dim3((n + MT - 1) / MT + E, (ff + 63) / 64), dim3(256), 0, stream,
+                       static_cast<const bf16_t*>(h), static_cast<size_t>(ldh), order, offsets, E, top, static_cast<const bf16_t*>(wg),
+                       static_cast<const bf16_t*>(wu), ff, width, limit, alpha, static_cast<bf16_t*>(y));
+    return dn_launch_status();
+  }
   hipLaunchKernelGGL(expert_up_kernel, dim3((n + TM - 1) / TM + E, (ff + TN - 1) / TN), dim3(256), 0, stream, h, h_dt,
                      static_cast<size_t>(ldh), order, offsets, E, top, wg, wu, w_dt, ff, width, limit, alpha, y, y_dt);
   return dn_launch_status();
@@ -273,6 +480,11 @@ int dn_moe_down(const void* y, int y_dt, const int* order, const int* offsets, i
                 int ff, float* out, hipStream_t stream) {
   if (!float_kind(y_dt) || !float_kind(w_dt)) return DN_ERR_DTYPE;
   if (n == 0) return 0;
+  if (y_dt == DN_BF16 && w_dt == DN_BF16 && ff % 32 == 0 && aligned16(y) && aligned16(wd)) {
+    hipLaunchKernelGGL(expert_down_mfma_kernel, dim3((n + MT - 1) / MT + E, (width + 63) / 64), dim3(256), 0, stream,
+                       static_cast<const bf16_t*>(y), order, offsets, E, static_cast<const bf16_t*>(wd), width, ff, out);
+    return dn_launch_status();
+  }
   hipLaunchKernelGGL(expert_down_kernel, dim3((n + TM - 1) / TM + E, (width + TN - 1) / TN), dim3(256), 0, stream, y, y_dt, order,
                      offsets, E, wd, w_dt, width, ff, out);
   return dn_launch_status();

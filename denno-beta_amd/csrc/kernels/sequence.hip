@@ -192,13 +192,18 @@ __global__ __launch_bounds__(256) void gated_kernel(const void* x, int x_dt, siz
 }
 
 // ---- the scan ----------------------------------------------------------------------------------------------
-// Per request, head and value column j a lane keeps column j of the head's state S [dk][dv] in registers and walks
-// the request's rows of this step in order:
+// Per request, head and 16 (or 4) value columns one wave keeps the head's state S [dk][those columns] in registers and
+// walks the request's rows of this step in order:
 //   a_i = key_from_decay ? 1 - w_i : k_i
 //   read_after:   S_i <- w_i S_i + a_i v_j ;  o_j = sum_i r_i S_i
 //   else:         o_j = sum_i r_i (S_i + u_i a_i v_j) ;  S_i <- w_i S_i + a_i v_j
-// The sum over i runs in ascending order, one fused multiply-add a step, whatever the step holds.  A row's r, k and w
-// reach the lanes through LDS; the next row's are asked for before the current row is worked on.
+// A column's key channels are shared out among KG lanes that lie side by side (4 lanes for heads of up to 32 key
+// channels, 16 beyond), so a wave has 64 / KG columns and a column's parts are joined inside a row of 16 lanes,
+// without LDS; a part's sum over i runs in ascending order, one fused multiply-add a step, and the parts are joined
+// in one fixed order, whatever the step holds.
+// A row's r, k and w reach the lanes through LDS, eight rows at a time; the next eight are asked for before the
+// current ones are worked on.  Places beyond a request's last row hold r = 0, a = 0, w = 1, which change nothing, so the
+// eight rows are worked on without a branch between them.
 struct ScanArgs {
   const float *r, *k, *v, *w, *u;
   size_t ldr, ldk, ldv, ldw;
@@ -210,72 +215,95 @@ struct ScanArgs {
   size_t ldo;
 };
 
-template <int DK>
+template <int DK, int KG, bool AFTER>
 __global__ __launch_bounds__(64) void scan_kernel(ScanArgs a) {
+  constexpr int KQ = DK / KG;
   constexpr int NL = DK >= 64 ? DK / 64 : 1;
-  __shared__ float sh[3 * DK];
-  __shared__ float shu[DK];
+  constexpr int TB = 8;      // rows asked for at a time: a trip to memory is paid once per eight rows, not per row
+  __shared__ __attribute__((aligned(16))) float sh[TB][3 * DK];
+  __shared__ __attribute__((aligned(16))) float shu[DK];
   const int s = blockIdx.z, h = blockIdx.y, lane = threadIdx.x;
-  const int j = blockIdx.x * 64 + lane;
+  const int kg = lane % KG, j = blockIdx.x * (64 / KG) + lane / KG;
   const int slot = a.slots[s];
   if (slot < 0) return;
   const int row0 = a.row_start[s], row1 = a.row_start[s + 1];
   if (row0 >= row1) return;
   const bool live = j < a.dv;
   const int dk = a.dk, dv = a.dv;
-  float* sp = a.state + static_cast<size_t>(slot) * a.slot_stride + static_cast<size_t>(h) * dk * dv + j;
-  float S[DK];
+  // the state lies [head][value column][key channel]: a lane's channels side by side, a column's lanes too
+  float* sp = a.state + static_cast<size_t>(slot) * a.slot_stride + (static_cast<size_t>(h) * dv + j) * dk + kg * KQ;
+  float S[KQ];
 #pragma unroll
-  for (int i = 0; i < DK; ++i) S[i] = (live && i < dk) ? sp[static_cast<size_t>(i) * dv] : 0.f;
+  for (int q = 0; q < KQ; ++q) S[q] = (live && kg * KQ + q < dk) ? sp[q] : 0.f;
   for (int i = lane; i < DK; i += 64) shu[i] = (a.u && i < dk) ? a.u[h * dk + i] : 0.f;
-  float nr[NL], nk[NL], nw[NL], nv;
-  auto fetch = [&](int t) {
+  float nr[TB][NL], nk[TB][NL], nw[TB][NL], nv[TB];
+  auto fetch = [&](int t0) {
 #pragma unroll
-    for (int q = 0; q < NL; ++q) {
-      const int i = lane + 64 * q;
-      const bool ok = i < dk;
-      nr[q] = ok ? a.r[t * a.ldr + h * dk + i] : 0.f;
-      nk[q] = (ok && !a.key_from_decay) ? a.k[t * a.ldk + h * dk + i] : 0.f;
-      nw[q] = ok ? a.w[t * a.ldw + h * dk + i] : 1.f;
+    for (int b = 0; b < TB; ++b) {
+      const int t = t0 + b;
+      const bool row = t < row1;
+#pragma unroll
+      for (int q = 0; q < NL; ++q) {
+        const int i = lane + 64 * q;
+        const bool ok = row && i < dk;
+        nr[b][q] = ok ? a.r[t * a.ldr + h * dk + i] : 0.f;
+        nk[b][q] = (ok && !a.key_from_decay) ? a.k[t * a.ldk + h * dk + i] : 0.f;
+        nw[b][q] = ok ? a.w[t * a.ldw + h * dk + i] : 1.f;
+      }
+      nv[b] = (row && live) ? a.v[t * a.ldv + h * dv + j] : 0.f;
     }
-    nv = live ? a.v[t * a.ldv + h * dv + j] : 0.f;
   };
   fetch(row0);
-  for (int t = row0; t < row1; ++t) {
+  for (int t0 = row0; t0 < row1; t0 += TB) {
+    float vj[TB];
 #pragma unroll
-    for (int q = 0; q < NL; ++q) {
-      const int i = lane + 64 * q;
-      if (i < DK) {
-        sh[i] = nr[q];
-        sh[DK + i] = a.key_from_decay ? 1.0f - nw[q] : nk[q];
-        sh[2 * DK + i] = nw[q];
+    for (int b = 0; b < TB; ++b) {
+#pragma unroll
+      for (int q = 0; q < NL; ++q) {
+        const int i = lane + 64 * q;
+        if (i < DK) {
+          sh[b][i] = nr[b][q];
+          sh[b][DK + i] = a.key_from_decay ? 1.0f - nw[b][q] : nk[b][q];
+          sh[b][2 * DK + i] = nw[b][q];
+        }
       }
+      vj[b] = nv[b];
     }
-    const float vj = nv;
     __syncthreads();
-    if (t + 1 < row1) fetch(t + 1);
-    float o = 0.f;
-    if (a.read_after) {
+    if (t0 + TB < row1) fetch(t0 + TB);
+    // (no branch inside the eight rows: their reads, sums and joins can then overlap)
+    float ob[TB];
 #pragma unroll
-      for (int i = 0; i < DK; ++i) {
-        S[i] = fmaf(sh[2 * DK + i], S[i], sh[DK + i] * vj);
-        o = fmaf(sh[i], S[i], o);
-      }
-    } else {
+    for (int b = 0; b < TB; ++b) {
+      const float* mr = sh[b] + kg * KQ;
+      const float* mk = mr + DK;
+      const float* mw = mk + DK;
+      const float* mu = shu + kg * KQ;
+      float o = 0.f;
 #pragma unroll
-      for (int i = 0; i < DK; ++i) {
-        const float kv = sh[DK + i] * vj;
-        o = fmaf(sh[i], fmaf(shu[i], kv, S[i]), o);
-        S[i] = fmaf(sh[2 * DK + i], S[i], kv);
+      for (int q = 0; q < KQ; ++q) {
+        const float kv = mk[q] * vj[b];
+        if (AFTER) {
+          S[q] = fmaf(mw[q], S[q], kv);
+          o = fmaf(mr[q], S[q], o);
+        } else {
+          o = fmaf(mr[q], fmaf(mu[q], kv, S[q]), o);
+          S[q] = fmaf(mw[q], S[q], kv);
+        }
       }
+      ob[b] = group_reduce<KG>(o, SumOp());
     }
-    if (live) a.out[t * a.ldo + h * dv + j] = o;
+    if (live && kg == 0) {
+#pragma unroll
+      for (int b = 0; b < TB; ++b)
+        if (t0 + b < row1) a.out[(t0 + b) * a.ldo + h * dv + j] = ob[b];
+    }
     __syncthreads();
   }
   if (live)
 #pragma unroll
-    for (int i = 0; i < DK; ++i)
-      if (i < dk) sp[static_cast<size_t>(i) * dv] = S[i];
+    for (int q = 0; q < KQ; ++q)
+      if (kg * KQ + q < dk) sp[q] = S[q];
 }
 
 // ---- a norm per head, with a gate ----------------------------------------------------------------------------
@@ -391,12 +419,19 @@ int dn_state_scan(const float* r, long long ldr, const float* k, long long ldk, 
   ScanArgs a{r, k, v, w, u, static_cast<size_t>(ldr), static_cast<size_t>(ldk), static_cast<size_t>(ldv), static_cast<size_t>(ldw),
              state, static_cast<size_t>(slot_stride), row_start, slots, H, dk, dv, read_after, key_from_decay, out,
              static_cast<size_t>(ldo)};
-  const dim3 grid((dv + 63) / 64, H, S);
-  if (dk <= 16) hipLaunchKernelGGL(scan_kernel<16>, grid, dim3(64), 0, stream, a);
-  else if (dk <= 32) hipLaunchKernelGGL(scan_kernel<32>, grid, dim3(64), 0, stream, a);
-  else if (dk <= 64) hipLaunchKernelGGL(scan_kernel<64>, grid, dim3(64), 0, stream, a);
-  else if (dk <= 128) hipLaunchKernelGGL(scan_kernel<128>, grid, dim3(64), 0, stream, a);
-  else hipLaunchKernelGGL(scan_kernel<256>, grid, dim3(64), 0, stream, a);
+  // (the parts of a column's sum by the head's size alone, never by the step: a row's bits are the same in every step)
+  const dim3 few((dv + 15) / 16, H, S), many((dv + 3) / 4, H, S);
+#define DN_SCAN(DK, KG, GRID)                                                                       \
+  do {                                                                                             \
+    if (read_after) hipLaunchKernelGGL((scan_kernel<DK, KG, true>), GRID, dim3(64), 0, stream, a); \
+    else hipLaunchKernelGGL((scan_kernel<DK, KG, false>), GRID, dim3(64), 0, stream, a);           \
+  } while (0)
+  if (dk <= 16) DN_SCAN(16, 4, few);
+  else if (dk <= 32) DN_SCAN(32, 4, few);
+  else if (dk <= 64) DN_SCAN(64, 16, many);
+  else if (dk <= 128) DN_SCAN(128, 16, many);
+  else DN_SCAN(256, 16, many);
+#undef DN_SCAN
   return dn_launch_status();
 }
 

@@ -1053,8 +1053,8 @@ def state_scan(r, k, v, w, u, state, row_start, slots, n_heads, dk, dv, out, rea
       a = 1 - w if key_from_decay else k
       read_after:  S <- diag(w) S + a v^T ;  o = S^T r
       else:        o = (S + diag(u) a v^T)^T r ;  S <- diag(w) S + a v^T        (u None: no bonus)
-    r, k, w: 32-bit [T, heads * dk]; v, out: 32-bit [T, heads * dv]; state: 32-bit [slots, heads * dk * dv], read and
-    written at the requests' slots."""
+    r, k, w: 32-bit [T, heads * dk]; v, out: 32-bit [T, heads * dv]; state: 32-bit [slots, heads * dv * dk] (a head's state
+    held [value column][key channel]), read and written at the requests' slots."""
     for t, name, n in ((r, "r", dk), (w, "w", dk), (v, "v", dv), (out, "out", dv)) + (() if key_from_decay else ((k, "k", dk),)):
         _dev(t, name, (torch.float32,), 2)
         _need(t.shape[1] == n_heads * n, lambda: f"state_scan: {name} {tuple(t.shape)}")

@@ -318,7 +318,7 @@ def gated(x, g, kind, out):
 def state_scan(r, k, v, w, u, state, row_start, slots, n_heads, dk, dv, out, read_after=False, key_from_decay=False):
     H = n_heads
     for slot, a, b in _requests(row_start, slots):
-        S = state[slot].view(H, dk, dv).clone()
+        S = state[slot].view(H, dv, dk).transpose(1, 2).clone()      # (held [head][value column][key channel])
         for t in range(a, b):
             rt, wt, vt = r[t].view(H, dk), w[t].view(H, dk), v[t].view(H, dv)
             at = (1.0 - wt) if key_from_decay else k[t].view(H, dk)
@@ -330,7 +330,7 @@ def state_scan(r, k, v, w, u, state, row_start, slots, n_heads, dk, dv, out, rea
                 bonus = kv * u.view(H, dk)[:, :, None] if u is not None else 0.0
                 out[t] = torch.einsum("hi,hij->hj", rt, S + bonus).reshape(-1)
                 S = wt[:, :, None] * S + kv
-        state[slot] = S.reshape(-1)
+        state[slot] = S.transpose(1, 2).reshape(-1)
     return out
 
 

@@ -149,7 +149,10 @@ def test_route_and_plan(T, E, top):
 
 
 @pytest.mark.parametrize("dtype", DT)
-@pytest.mark.parametrize("T,E,top,ff,width", [(1, 3, 2, 8, 24), (45, 6, 3, 70, 50), (300, 4, 1, 33, 96)])
+# (bfloat16 with a width and an inner size that are multiples of 32 takes the matrix-core kernels; tiles of 64 places with
+# one row, with a last block that is not full, experts that nobody chose)
+@pytest.mark.parametrize("T,E,top,ff,width", [(1, 3, 2, 8, 24), (45, 6, 3, 70, 50), (300, 4, 1, 33, 96), (200, 5, 2, 64, 128),
+                                              (9, 8, 2, 96, 64), (77, 3, 3, 40, 32), (3, 40, 2, 32, 160)])
 def test_experts(dtype, T, E, top, ff, width):
     h = torch.randn(T, width, device=DEV).to(dtype)
     wg, wu = ((torch.randn(E, ff, width, device=DEV) / width ** 0.5).to(dtype) for _ in range(2))
@@ -173,6 +176,18 @@ def test_experts(dtype, T, E, top, ff, width):
     ops.moe_combine(out, wts, x)
     ref.moe_combine(out.cpu(), wts.cpu(), hx)
     close(x, hx)
+
+
+@pytest.mark.parametrize("T,H,N,K", [(1, 2, 24, 32), (130, 3, 70, 64), (65, 1, 33, 96)])
+def test_heads_linear_on_the_matrix_cores(T, H, N, K):
+    """bfloat16 rows at offsets that are multiples of 8 numbers: the kernel of 16 x 16 x 32 blocks."""
+    a = torch.randn(T, 8 + H * (K + 8), device=DEV).bfloat16()
+    w = (torch.randn(H, N, K, device=DEV) / K ** 0.5).bfloat16()
+    for dtype in DT:
+        both("heads_linear", lambda: (a, w, torch.zeros(T, 2 + H * (N + 1), dtype=dtype, device=DEV), 8, K + 8, 2, N + 1), [2], dtype)
+    one = ops.heads_linear(a[T // 2:T // 2 + 1].contiguous(), w, torch.zeros(1, 2 + H * (N + 1), device=DEV), 8, K + 8, 2, N + 1)
+    many = ops.heads_linear(a, w, torch.zeros(T, 2 + H * (N + 1), device=DEV), 8, K + 8, 2, N + 1)
+    assert torch.equal(many[T // 2:T // 2 + 1], one), "a row's sums depend on the rows beside it"
 
 
 def test_a_row_does_not_depend_on_its_neighbours():
