@@ -282,38 +282,61 @@ constexpr int MT = 64;      // rows of a workgroup's tile
 __device__ __forceinline__ bf16x8 load8(const bf16_t* p) { return *reinterpret_cast<const bf16x8*>(p); }
 
 // acc[i][j] += A[rows i] . W[cols j]^T over K; a_ptr[i], w_ptr[j]: this lane's row of block i / column of block j, at
-// its own k offset
-template <bool DUAL>
-__device__ __forceinline__ void mfma_tile(const bf16_t* const a_ptr[2], const bf16_t* const w_ptr[2], const bf16_t* const w2_ptr[2],
-                                          int K, f32x4 acc[2][2], f32x4 acc2[2][2]) {
+// its own k offset.  PACKED: W lies in blocks of 16 columns x 32 of K in the lanes' own order (dn_pack_matrix): w_ptr[j]
+// is the lane's 16 bytes of the column block's first step, a step further 512 numbers on; a load is then 1 KB in one
+// piece, where from rows it touches 16 cache lines per 16 lanes, and the rate of those lookups is what bounds the kernel.
+template <bool DUAL, bool PACKED, int CB>
+__device__ __forceinline__ void mfma_tile(const bf16_t* const a_ptr[2], const bf16_t* const w_ptr[CB], const bf16_t* const w2_ptr[CB],
+                                          int K, f32x4 acc[2][CB], f32x4 acc2[2][CB]) {
+  constexpr int WSTEP = PACKED ? 512 : 32;
 #pragma unroll 2
   for (int k0 = 0; k0 < K; k0 += 32) {
-    bf16x8 af[2], wf[2], wf2[2];
+    bf16x8 af[2], wf[CB], wf2[CB];
 #pragma unroll
     for (int i = 0; i < 2; ++i) af[i] = load8(a_ptr[i] + k0);
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      wf[j] = load8(w_ptr[j] + k0);
-      if (DUAL) wf2[j] = load8(w2_ptr[j] + k0);
+    for (int j = 0; j < CB; ++j) {
+      wf[j] = load8(w_ptr[j] + static_cast<size_t>(k0 / 32) * WSTEP);
+      if (DUAL) wf2[j] = load8(w2_ptr[j] + static_cast<size_t>(k0 / 32) * WSTEP);
     }
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
-      for (int j = 0; j < 2; ++j) {
+      for (int j = 0; j < CB; ++j) {
         acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[j], af[i], acc[i][j], 0, 0, 0);
         if (DUAL) acc2[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf2[j], af[i], acc2[i][j], 0, 0, 0);
       }
   }
 }
 
-// which expert and which of its tiles of 64 places workgroup `id` has
+// Workgroups are handed to the eight XCDs in turn, and each XCD has an L2 of its own: the launch is one line of
+// workgroups, and workgroup L takes the work L' = (L % 8) * (n / 8) + L / 8, so that an XCD gets a run of neighbouring
+// tiles (row tiles fastest: the tiles of one expert and column block, which read the same weights, meet in one L2).
+// n: the launch's size, a multiple of 8; -> (row tile, column tile), or row tile -1 beyond `tiles_x * tiles_y`.
+__device__ __forceinline__ void xcd_tile(int tiles_x, int tiles_y, int& tx, int& ty) {
+  const int n = gridDim.x, L = blockIdx.x;
+  const int at = (L % 8) * (n / 8) + L / 8;
+  tx = at < tiles_x * tiles_y ? at % tiles_x : -1;
+  ty = at / tiles_x;
+}
+
+// which expert and which of its tiles of 64 places workgroup `id` has.  The experts' offsets come to LDS in one
+// parallel load first (a walk through them in memory is a chain of dependent loads, as long as the tile's own work).
+constexpr int OFFSETS_IN_LDS = 1024;
 __device__ __forceinline__ bool expert_tile64(const int* offsets, int E, int id, int& e, int& p0, int& p1) {
+  __shared__ int held[OFFSETS_IN_LDS + 1];
+  const bool in_lds = E <= OFFSETS_IN_LDS;
+  if (in_lds) {
+    for (int i = threadIdx.x; i <= E; i += blockDim.x) held[i] = offsets[i];
+    __syncthreads();
+  }
+  const int* off = in_lds ? held : offsets;
   for (e = 0; e < E; ++e) {
-    const int cnt = offsets[e + 1] - offsets[e];
+    const int cnt = off[e + 1] - off[e];
     const int tiles = (cnt + MT - 1) / MT;
     if (id < tiles) {
-      p0 = offsets[e] + id * MT;
-      p1 = min(p0 + MT, offsets[e + 1]);
+      p0 = off[e] + id * MT;
+      p1 = min(p0 + MT, off[e + 1]);
       return true;
     }
     id -= tiles;
@@ -323,11 +346,12 @@ __device__ __forceinline__ bool expert_tile64(const int* offsets, int E, int id,
 
 __global__ __launch_bounds__(256) void expert_up_mfma_kernel(const bf16_t* h, size_t ldh, const int* order, const int* offsets, int E,
                                                              int top, const bf16_t* wg, const bf16_t* wu, int ff, int width,
-                                                             float limit, float alpha, bf16_t* y) {
-  int e, p0, p1;
-  if (!expert_tile64(offsets, E, blockIdx.x, e, p0, p1)) return;
+                                                             float limit, float alpha, bf16_t* y, int tiles_x) {
+  int e, p0, p1, tx, ty;
+  xcd_tile(tiles_x, (ff + 63) / 64, tx, ty);
+  if (tx < 0 || !expert_tile64(offsets, E, tx, e, p0, p1)) return;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int pw = p0 + (wave >> 1) * 32, nw = blockIdx.y * 64 + (wave & 1) * 32;
+  const int pw = p0 + (wave >> 1) * 32, nw = ty * 64 + (wave & 1) * 32;
   if (pw >= p1 || nw >= ff) return;
   const int kq = (lane >> 4) * 8, lr = lane & 15;
   const bf16_t *a_ptr[2], *g_ptr[2], *u_ptr[2];
@@ -340,7 +364,7 @@ __global__ __launch_bounds__(256) void expert_up_mfma_kernel(const bf16_t* h, si
     u_ptr[i] = wu + (static_cast<size_t>(e) * ff + n) * width + kq;
   }
   f32x4 g[2][2] = {}, u[2][2] = {};
-  mfma_tile<true>(a_ptr, g_ptr, u_ptr, width, g, u);
+  mfma_tile<true, false, 2>(a_ptr, g_ptr, u_ptr, width, g, u);
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
     const int p = pw + 16 * i + lr;
@@ -359,11 +383,12 @@ __global__ __launch_bounds__(256) void expert_up_mfma_kernel(const bf16_t* h, si
 }
 
 __global__ __launch_bounds__(256) void expert_down_mfma_kernel(const bf16_t* y, const int* order, const int* offsets, int E,
-                                                               const bf16_t* wd, int width, int ff, float* out) {
-  int e, p0, p1;
-  if (!expert_tile64(offsets, E, blockIdx.x, e, p0, p1)) return;
+                                                               const bf16_t* wd, int width, int ff, float* out, int tiles_x) {
+  int e, p0, p1, tx, ty;
+  xcd_tile(tiles_x, (width + 63) / 64, tx, ty);
+  if (tx < 0 || !expert_tile64(offsets, E, tx, e, p0, p1)) return;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int pw = p0 + (wave >> 1) * 32, nw = blockIdx.y * 64 + (wave & 1) * 32;
+  const int pw = p0 + (wave >> 1) * 32, nw = ty * 64 + (wave & 1) * 32;
   if (pw >= p1 || nw >= width) return;
   const int kq = (lane >> 4) * 8, lr = lane & 15;
   const bf16_t *a_ptr[2], *w_ptr[2];
@@ -373,7 +398,7 @@ __global__ __launch_bounds__(256) void expert_down_mfma_kernel(const bf16_t* y, 
     w_ptr[i] = wd + (static_cast<size_t>(e) * width + min(nw + 16 * i + lr, width - 1)) * ff + kq;
   }
   f32x4 acc[2][2] = {};
-  mfma_tile<false>(a_ptr, w_ptr, nullptr, ff, acc, nullptr);
+  mfma_tile<false, false, 2>(a_ptr, w_ptr, nullptr, ff, acc, nullptr);
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
     const int p = pw + 16 * i + lr;
@@ -385,6 +410,78 @@ __global__ __launch_bounds__(256) void expert_down_mfma_kernel(const bf16_t* y, 
 #pragma unroll
       for (int r = 0; r < 4; ++r)
         if (n + r < width) out[pair * width + n + r] = acc[i][j][r];
+    }
+  }
+}
+
+
+// The same two kernels for packed weights (the experts' matrices stacked and packed as one; an expert's rows start at a
+// multiple of 16): a wave takes 32 pairs x 64 columns, a workgroup 64 x 128.
+__global__ __launch_bounds__(256) void expert_up_packed_kernel(const bf16_t* h, size_t ldh, const int* order, const int* offsets, int E,
+                                                               int top, const bf16_t* wg, const bf16_t* wu, int ff, int width,
+                                                               float limit, float alpha, bf16_t* y, int tiles_x) {
+  int e, p0, p1, tx, ty;
+  xcd_tile(tiles_x, (ff + 127) / 128, tx, ty);
+  if (tx < 0 || !expert_tile64(offsets, E, tx, e, p0, p1)) return;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int pw = p0 + (wave >> 1) * 32, nw = ty * 128 + (wave & 1) * 64;
+  if (pw >= p1 || nw >= ff) return;
+  const int kq = (lane >> 4) * 8, lr = lane & 15, ksteps = width / 32;
+  const bf16_t *a_ptr[2], *g_ptr[4], *u_ptr[4];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) a_ptr[i] = h + static_cast<size_t>(order[min(pw + 16 * i + lr, p1 - 1)] / top) * ldh + kq;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const size_t block = (static_cast<size_t>(e) * ff + min(nw + 16 * j, ff - 16)) / 16;
+    g_ptr[j] = wg + block * ksteps * 512 + lane * 8;
+    u_ptr[j] = wu + block * ksteps * 512 + lane * 8;
+  }
+  f32x4 g[2][4] = {}, u[2][4] = {};
+  mfma_tile<true, true, 4>(a_ptr, g_ptr, u_ptr, width, g, u);
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int p = pw + 16 * i + lr;
+    if (p >= p1) continue;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int n = nw + 16 * j + (lane >> 4) * 4;
+      if (n >= ff) continue;      // (ff is a multiple of 16: a block is whole or absent)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const float gv = fminf(g[i][j][r], limit), uv = fminf(fmaxf(u[i][j][r], -limit), limit);
+        y[static_cast<size_t>(p) * ff + n + r] = from_float<bf16_t>(gv / (1.0f + expf(-alpha * gv)) * (uv + 1.0f));
+      }
+    }
+  }
+}
+
+__global__ __launch_bounds__(256) void expert_down_packed_kernel(const bf16_t* y, const int* order, const int* offsets, int E,
+                                                                 const bf16_t* wd, int width, int ff, float* out, int tiles_x) {
+  int e, p0, p1, tx, ty;
+  xcd_tile(tiles_x, (width + 127) / 128, tx, ty);
+  if (tx < 0 || !expert_tile64(offsets, E, tx, e, p0, p1)) return;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int pw = p0 + (wave >> 1) * 32, nw = ty * 128 + (wave & 1) * 64;
+  if (pw >= p1 || nw >= width) return;
+  const int kq = (lane >> 4) * 8, lr = lane & 15, ksteps = ff / 32;
+  const bf16_t *a_ptr[2], *w_ptr[4];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) a_ptr[i] = y + static_cast<size_t>(min(pw + 16 * i + lr, p1 - 1)) * ff + kq;
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+    w_ptr[j] = wd + (static_cast<size_t>(e) * width + min(nw + 16 * j, width - 16)) / 16 * ksteps * 512 + lane * 8;
+  f32x4 acc[2][4] = {};
+  mfma_tile<false, true, 4>(a_ptr, w_ptr, nullptr, ff, acc, nullptr);
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int p = pw + 16 * i + lr;
+    if (p >= p1) continue;
+    const size_t pair = order[p];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int n = nw + 16 * j + (lane >> 4) * 4;
+      if (n >= width) continue;
+      *reinterpret_cast<f32x4*>(out + pair * width + n) = acc[i][j];
     }
   }
 }
@@ -404,7 +501,7 @@ __global__ __launch_bounds__(256) void heads_linear_mfma_kernel(const bf16_t* A,
     w_ptr[i] = W + (static_cast<size_t>(hd) * N + min(nw + 16 * i + lr, N - 1)) * K + kq;
   }
   f32x4 acc[2][2] = {};
-  mfma_tile<false>(a_ptr, w_ptr, nullptr, K, acc, nullptr);
+  mfma_tile<false, false, 2>(a_ptr, w_ptr, nullptr, K, acc, nullptr);
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
     const int t = tw + 16 * i + lr;
@@ -461,14 +558,25 @@ int dn_moe_plan(const int* ids, int n, int E, int* offsets, int* order, hipStrea
 }
 
 int dn_moe_up(const void* h, int h_dt, long long ldh, const int* order, const int* offsets, int E, int top, int n, const void* wg,
-              const void* wu, int w_dt, int ff, int width, float limit, float alpha, void* y, int y_dt, hipStream_t stream) {
+              const void* wu, int w_dt, int ff, int width, float limit, float alpha, void* y, int y_dt, int packed,
+              hipStream_t stream) {
   if (!float_kind(h_dt) || !float_kind(w_dt) || !float_kind(y_dt)) return DN_ERR_DTYPE;
   if (n == 0) return 0;
+  if (packed) {
+    if (h_dt != DN_BF16 || w_dt != DN_BF16 || y_dt != DN_BF16) return DN_ERR_DTYPE;
+    if (width % 32 != 0 || ff % 16 != 0 || ldh % 8 != 0 || !aligned16(h) || !aligned16(wg) || !aligned16(wu)) return DN_ERR_SHAPE;
+    const int tiles_x = (n + MT - 1) / MT + E, tiles = tiles_x * ((ff + 127) / 128);
+    hipLaunchKernelGGL(expert_up_packed_kernel, dim3((tiles + 7) / 8 * 8), dim3(256), 0, stream, static_cast<const bf16_t*>(h),
+                       static_cast<size_t>(ldh), order, offsets, E, top, static_cast<const bf16_t*>(wg), static_cast<const bf16_t*>(wu),
+                       ff, width, limit, alpha, static_cast<bf16_t*>(y), tiles_x);
+    return dn_launch_status();
+  }
   if (h_dt == DN_BF16 && w_dt == DN_BF16 && y_dt == DN_BF16 && width % 32 == 0 && ldh % 8 == 0 && aligned16(h) && aligned16(wg) &&
       aligned16(wu)) {
-    hipLaunchKernelGGL(expert_up_mfma_kernel, dim3((n + MT - 1) / MT + E, (ff + 63) / 64), dim3(256), 0, stream,
+    const int tiles_x = (n + MT - 1) / MT + E, tiles = tiles_x * ((ff + 63) / 64);
+    hipLaunchKernelGGL(expert_up_mfma_kernel, dim3((tiles + 7) / 8 * 8), dim3(256), 0, stream,
                        static_cast<const bf16_t*>(h), static_cast<size_t>(ldh), order, offsets, E, top, static_cast<const bf16_t*>(wg),
-                       static_cast<const bf16_t*>(wu), ff, width, limit, alpha, static_cast<bf16_t*>(y));
+                       static_cast<const bf16_t*>(wu), ff, width, limit, alpha, static_cast<bf16_t*>(y), tiles_x);
     return dn_launch_status();
   }
   hipLaunchKernelGGL(expert_up_kernel, dim3((n + TM - 1) / TM + E, (ff + TN - 1) / TN), dim3(256), 0, stream, h, h_dt,
@@ -477,12 +585,21 @@ int dn_moe_up(const void* h, int h_dt, long long ldh, const int* order, const in
 }
 
 int dn_moe_down(const void* y, int y_dt, const int* order, const int* offsets, int E, int n, const void* wd, int w_dt, int width,
-                int ff, float* out, hipStream_t stream) {
+                int ff, float* out, int packed, hipStream_t stream) {
   if (!float_kind(y_dt) || !float_kind(w_dt)) return DN_ERR_DTYPE;
   if (n == 0) return 0;
+  if (packed) {
+    if (y_dt != DN_BF16 || w_dt != DN_BF16) return DN_ERR_DTYPE;
+    if (ff % 32 != 0 || width % 16 != 0 || !aligned16(y) || !aligned16(wd) || !aligned16(out)) return DN_ERR_SHAPE;
+    const int tiles_x = (n + MT - 1) / MT + E, tiles = tiles_x * ((width + 127) / 128);
+    hipLaunchKernelGGL(expert_down_packed_kernel, dim3((tiles + 7) / 8 * 8), dim3(256), 0, stream, static_cast<const bf16_t*>(y),
+                       order, offsets, E, static_cast<const bf16_t*>(wd), width, ff, out, tiles_x);
+    return dn_launch_status();
+  }
   if (y_dt == DN_BF16 && w_dt == DN_BF16 && ff % 32 == 0 && aligned16(y) && aligned16(wd)) {
-    hipLaunchKernelGGL(expert_down_mfma_kernel, dim3((n + MT - 1) / MT + E, (width + 63) / 64), dim3(256), 0, stream,
-                       static_cast<const bf16_t*>(y), order, offsets, E, static_cast<const bf16_t*>(wd), width, ff, out);
+    const int tiles_x = (n + MT - 1) / MT + E, tiles = tiles_x * ((width + 63) / 64);
+    hipLaunchKernelGGL(expert_down_mfma_kernel, dim3((tiles + 7) / 8 * 8), dim3(256), 0, stream,
+                       static_cast<const bf16_t*>(y), order, offsets, E, static_cast<const bf16_t*>(wd), width, ff, out, tiles_x);
     return dn_launch_status();
   }
   hipLaunchKernelGGL(expert_down_kernel, dim3((n + TM - 1) / TM + E, (width + TN - 1) / TN), dim3(256), 0, stream, y, y_dt, order,

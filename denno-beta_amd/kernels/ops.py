@@ -139,8 +139,8 @@ def _declare(name, lib):
             "dn_heads_linear": [P, I, c_longlong, I, I, P, I, P, I, c_longlong, I, I, I, I, I, I, P],
             "dn_moe_route": [P, P, I, I, I, P, P, P],
             "dn_moe_plan": [P, I, I, P, P, P],
-            "dn_moe_up": [P, I, c_longlong, P, P, I, I, I, P, P, I, I, I, F, F, P, I, P],
-            "dn_moe_down": [P, I, P, P, I, I, P, I, I, I, P, P],
+            "dn_moe_up": [P, I, c_longlong, P, P, I, I, I, P, P, I, I, I, F, F, P, I, I, P],
+            "dn_moe_down": [P, I, P, P, I, I, P, I, I, I, P, I, P],
             "dn_moe_combine": [P, P, I, I, I, P, c_longlong, P],
         },
         "sampling": {
@@ -1131,28 +1131,54 @@ def moe_plan(ids, n_experts, offsets, order):
     _ok(_lib("grouped").dn_moe_plan(ids.data_ptr(), n, n_experts, offsets.data_ptr(), order.data_ptr(), _stream()), "moe_plan")
 
 
-def moe_up(h, order, offsets, top, w_gate, w_up, limit, alpha, y):
+def experts_packable(n_experts, rows, inner):
+    """Whether stacked expert matrices [experts * rows, inner] can be held packed for the matrix cores (pack_matrix on
+    the stack): an expert's rows start at a block of 16, the inner size is whole steps of 32."""
+    return rows % 16 == 0 and inner % 32 == 0
+
+
+def moe_up(h, order, offsets, top, w_gate, w_up, limit, alpha, y, dims=None):
     """For place p of expert e, the row t = order[p] // top: g = min(w_gate[e] h[t], limit), u = clamp(w_up[e] h[t], -limit,
-    limit), y[p] = g * sigmoid(alpha * g) * (u + 1).  w_gate, w_up: [experts, ff, width]; y [T * top, ff]."""
-    _dev(h, "h", _FLOATS, 2), _dev(w_gate, "w_gate", _FLOATS, 3), _dev(w_up, "w_up", (w_gate.dtype,), 3), _dev(y, "y", _FLOATS, 2)
-    E, ff, width = w_gate.shape
+    limit), y[p] = g * sigmoid(alpha * g) * (u + 1).  w_gate, w_up: [experts, ff, width]; y [T * top, ff].
+    dims = (experts, ff, width): w_gate and w_up are PackedMatrix of the stacked [experts * ff, width] (experts_packable)."""
+    _dev(h, "h", _FLOATS, 2), _dev(y, "y", _FLOATS, 2)
     n = order.shape[0]
-    _need(w_gate.is_contiguous() and w_up.is_contiguous() and tuple(w_up.shape) == (E, ff, width) and h.shape[1] == width
-          and y.is_contiguous() and tuple(y.shape) == (n, ff) and offsets.shape[0] == E + 1 and n == h.shape[0] * top, "moe_up: shapes")
+    if dims is not None:
+        E, ff, width = dims
+        _need(isinstance(w_gate, PackedMatrix) and isinstance(w_up, PackedMatrix) and tuple(w_gate.shape) == (E * ff, width)
+              and tuple(w_up.shape) == (E * ff, width) and experts_packable(E, ff, width), "moe_up: packed weights")
+        wdt = torch.bfloat16
+    else:
+        _dev(w_gate, "w_gate", _FLOATS, 3), _dev(w_up, "w_up", (w_gate.dtype,), 3)
+        E, ff, width = w_gate.shape
+        _need(w_gate.is_contiguous() and w_up.is_contiguous() and tuple(w_up.shape) == (E, ff, width), "moe_up: weights")
+        wdt = w_gate.dtype
+    _need(h.shape[1] == width and y.is_contiguous() and tuple(y.shape) == (n, ff) and offsets.shape[0] == E + 1
+          and n == h.shape[0] * top, "moe_up: shapes")
     _ok(_lib("grouped").dn_moe_up(h.data_ptr(), _CODE[h.dtype], _rows(h, "h"), order.data_ptr(), offsets.data_ptr(), E, top, n,
-                                  w_gate.data_ptr(), w_up.data_ptr(), _CODE[w_gate.dtype], ff, width, float(limit), float(alpha),
-                                  y.data_ptr(), _CODE[y.dtype], _stream()), "moe_up")
+                                  w_gate.data_ptr(), w_up.data_ptr(), _CODE[wdt], ff, width, float(limit), float(alpha),
+                                  y.data_ptr(), _CODE[y.dtype], int(dims is not None), _stream()), "moe_up")
 
 
-def moe_down(y, order, offsets, w_down, out):
-    """out[order[p], :] = w_down[e] y[p, :] for the places p of expert e; w_down [experts, width, ff]; out 32-bit [T * top, width]."""
-    _dev(y, "y", _FLOATS, 2), _dev(w_down, "w_down", _FLOATS, 3), _dev(out, "out", (torch.float32,), 2)
-    E, width, ff = w_down.shape
+def moe_down(y, order, offsets, w_down, out, dims=None):
+    """out[order[p], :] = w_down[e] y[p, :] for the places p of expert e; w_down [experts, width, ff]; out 32-bit [T * top, width].
+    dims = (experts, width, ff): w_down is a PackedMatrix of the stacked [experts * width, ff]."""
+    _dev(y, "y", _FLOATS, 2), _dev(out, "out", (torch.float32,), 2)
     n = order.shape[0]
-    _need(w_down.is_contiguous() and y.is_contiguous() and tuple(y.shape) == (n, ff) and out.is_contiguous()
-          and tuple(out.shape) == (n, width) and offsets.shape[0] == E + 1, "moe_down: shapes")
+    if dims is not None:
+        E, width, ff = dims
+        _need(isinstance(w_down, PackedMatrix) and tuple(w_down.shape) == (E * width, ff) and experts_packable(E, width, ff),
+              "moe_down: packed weights")
+        wdt = torch.bfloat16
+    else:
+        _dev(w_down, "w_down", _FLOATS, 3)
+        E, width, ff = w_down.shape
+        _need(w_down.is_contiguous(), "moe_down: weights")
+        wdt = w_down.dtype
+    _need(y.is_contiguous() and tuple(y.shape) == (n, ff) and out.is_contiguous() and tuple(out.shape) == (n, width)
+          and offsets.shape[0] == E + 1, "moe_down: shapes")
     _ok(_lib("grouped").dn_moe_down(y.data_ptr(), _CODE[y.dtype], order.data_ptr(), offsets.data_ptr(), E, n, w_down.data_ptr(),
-                                    _CODE[w_down.dtype], width, ff, out.data_ptr(), _stream()), "moe_down")
+                                    _CODE[wdt], width, ff, out.data_ptr(), int(dims is not None), _stream()), "moe_down")
 
 
 def moe_combine(out, wts, x):

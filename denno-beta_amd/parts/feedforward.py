@@ -111,10 +111,22 @@ class RoutedExperts(Part):
         self.w_up = tensors[self.templates["up"].format(e="*")].view(E, self.inner, self.width)
         self.w_down = tensors[self.templates["down"].format(e="*")].view(E, self.width, self.inner)
         self.correction = tensors[self.correction_name] if self.correction_name else None
+        # bfloat16 experts on the GPU are held packed for the matrix cores, the stack as one matrix, where an expert's
+        # rows start at a block's border (the rows they came from are not kept)
+        self.up_dims = self.down_dims = None
+        if self.w_gate.dtype == torch.bfloat16 and self.w_gate.is_cuda:
+            if ops.experts_packable(E, self.inner, self.width):
+                self.w_gate = ops.pack_matrix(self.w_gate.view(E * self.inner, self.width))
+                self.w_up = ops.pack_matrix(self.w_up.view(E * self.inner, self.width))
+                self.up_dims = (E, self.inner, self.width)
+            if ops.experts_packable(E, self.width, self.inner):
+                self.w_down = ops.pack_matrix(self.w_down.view(E * self.width, self.inner))
+                self.down_dims = (E, self.width, self.inner)
+        self.w_dtype = torch.bfloat16 if isinstance(self.w_gate, ops.PackedMatrix) else self.w_gate.dtype
 
     def forward(self, h, ctx, accumulate_into):
         T, top, dev = h.shape[0], self.top, h.device
-        wdt = self.w_gate.dtype
+        wdt = self.w_dtype
         if h.dtype != wdt:        # (experts stored in 32-bit in a bfloat16 engine: their products run on widened rows)
             h = ops.cast(h.contiguous(), torch.empty(h.shape, dtype=wdt, device=dev))
         z = self.router(h, out_dtype=torch.float32)
@@ -125,7 +137,7 @@ class RoutedExperts(Part):
         order = torch.empty(T * top, dtype=torch.int32, device=dev)
         ops.moe_plan(ids, self.n_experts, offsets, order)
         y = torch.empty((T * top, self.inner), dtype=wdt, device=dev)
-        ops.moe_up(h, order, offsets, top, self.w_gate, self.w_up, self.limit, self.alpha, y)
+        ops.moe_up(h, order, offsets, top, self.w_gate, self.w_up, self.limit, self.alpha, y, dims=self.up_dims)
         out = torch.empty((T * top, self.width), dtype=torch.float32, device=dev)
-        ops.moe_down(y, order, offsets, self.w_down, out)
+        ops.moe_down(y, order, offsets, self.w_down, out, dims=self.down_dims)
         ops.moe_combine(out, wts, accumulate_into)

@@ -213,7 +213,7 @@ class DecoderModel:
                 for v in vars(p).values():
                     if isinstance(v, Linear):
                         add(v.weight), add(v.bias)
-                    elif isinstance(v, torch.Tensor):
+                    elif isinstance(v, (torch.Tensor, ops.PackedMatrix)):
                         add(v)
         add(self.head.weight)
         add(getattr(self.final_norm, "weight", None)), add(getattr(self.final_norm, "bias", None))

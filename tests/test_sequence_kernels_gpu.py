@@ -152,7 +152,7 @@ def test_route_and_plan(T, E, top):
 # (bfloat16 with a width and an inner size that are multiples of 32 takes the matrix-core kernels; tiles of 64 places with
 # one row, with a last block that is not full, experts that nobody chose)
 @pytest.mark.parametrize("T,E,top,ff,width", [(1, 3, 2, 8, 24), (45, 6, 3, 70, 50), (300, 4, 1, 33, 96), (200, 5, 2, 64, 128),
-                                              (9, 8, 2, 96, 64), (77, 3, 3, 40, 32), (3, 40, 2, 32, 160)])
+                                              (9, 8, 2, 96, 64), (77, 3, 3, 40, 32), (3, 40, 2, 32, 160), (150, 4, 2, 160, 192), (70, 2, 2, 16, 32)])
 def test_experts(dtype, T, E, top, ff, width):
     h = torch.randn(T, width, device=DEV).to(dtype)
     wg, wu = ((torch.randn(E, ff, width, device=DEV) / width ** 0.5).to(dtype) for _ in range(2))
@@ -170,6 +170,15 @@ def test_experts(dtype, T, E, top, ff, width):
     ho = torch.zeros(T * top, width)
     ref.moe_down(y.cpu(), order.cpu(), offsets.cpu(), wd.cpu(), ho)
     close(out, ho, dtype, "moe_down")
+    if dtype == torch.bfloat16 and ops.experts_packable(E, ff, width) and ops.experts_packable(E, width, ff):
+        # the experts' matrices stacked and packed for the matrix cores: the same numbers
+        pg, pu = ops.pack_matrix(wg.view(E * ff, width)), ops.pack_matrix(wu.view(E * ff, width))
+        y2 = torch.zeros_like(y)
+        ops.moe_up(h, order, offsets, top, pg, pu, 1.5, 1.702, y2, dims=(E, ff, width))
+        close(y2, hy, dtype, "moe_up, packed")
+        out2 = torch.zeros_like(out)
+        ops.moe_down(y, order, offsets, ops.pack_matrix(wd.view(E * width, ff)), out2, dims=(E, width, ff))
+        close(out2, ho, dtype, "moe_down, packed")
     wts = torch.rand(T, top, device=DEV)
     x = torch.randn(T, width, device=DEV)
     hx = x.cpu().clone()
