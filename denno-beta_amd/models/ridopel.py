@@ -26,7 +26,7 @@ from ..parts.model import DecoderSpec, LayerCall, LayerSpec
 
 MIXER_TYPES = ("latent_attention", "wkv", "hgrn2")
 EXPERT_ALPHA = 1.702
-DEFAULT_MAX_POSITIONS = 32768
+DEFAULT_MAX_POSITIONS = 65536
 DEFAULT_DECAY_RANK = 32        # for weights made here; a checkpoint's own tensors say theirs
 
 
