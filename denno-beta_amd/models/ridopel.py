@@ -4,7 +4,8 @@ config.json: `vocab`, `width`, `norm.eps`, `canon.taps` (absent: no input convol
 `layers` (each: `type`, `mixer` with the mixer's sizes, `mlp` or null) and `loop` (`start`, `stop`, `times`; absent: every
 layer runs once).  Optional: `max_positions` (the engine's limit on a request's length; the architecture itself has
 none) and, in a wkv mixer, `decay_rank` (the inner size of the decay's two small matrices, which a checkpoint's tensors
-give by their shape).
+give by their shape) and, in a latent_attention mixer, `keep` ("latent" or "heads": what the cache holds, see
+parts.mixers.LatentAttention; absent: the latent where the attention kernels take its width).
 
 The model: token rows, normed; then the layers in their order, layers start .. stop - 1 `times` times in a row with the
 same weights and a cache of their own per pass; before the first layer of every pass the stream becomes
@@ -153,7 +154,7 @@ def _mixer(cfg: RidopelConfig, i: int, layer: dict):
     if layer["type"] == "latent_attention":
         return ("latent_attention", dict(
             width=W, n_heads=m["heads"], head_dim=m["dim"], rot_dim=m["rot_dim"], value_dim=m["vdim"], kv_rank=m["kv_rank"],
-            scale=m["scale"], eps=cfg.eps, position=dict(dims=m["rot"]["dims"], base=m["rot"]["base"]),
+            scale=m["scale"], eps=cfg.eps, position=dict(dims=m["rot"]["dims"], base=m["rot"]["base"]), keep=m.get("keep"),
             names=dict(q=p + "q", dkv=p + "dkv", g=p + "g", uk=p + "uk", uv=p + "uv", o=p + "o", dkv_norm=p + "dkv.norm")))
     if layer["type"] == "wkv":
         names = {s: p + s for s in ("r", "k", "v", "g", "w1", "w2", "o", "w0", "u", "norm")}

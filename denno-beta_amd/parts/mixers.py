@@ -118,13 +118,21 @@ class LatentAttention(Part):
     libraries = ("sequence", "grouped")
 
     def __init__(self, width: int, n_heads: int, head_dim: int, rot_dim: int, value_dim: int, kv_rank: int, scale: float,
-                 eps: float, position: dict, names: dict):
-        """names: q, dkv, g, uk, uv, o (matrices); dkv_norm (vector)."""
+                 eps: float, position: dict, names: dict, keep: str = None):
+        """names: q, dkv, g, uk, uv, o (matrices); dkv_norm (vector).
+        keep: "latent" (the form above), "heads" (every head's own key [W_uk c | turned part] and value W_uv c are kept,
+        as an ordinary attention does: more cache, and the way out where kv_rank + rot_dim is beyond the attention kernels'
+        largest head), or None: "latent" where it fits."""
         self.width, self.n_heads, self.head_dim, self.rot_dim = width, n_heads, head_dim, rot_dim
         self.value_dim, self.kv_rank, self.scale, self.eps, self.names = value_dim, kv_rank, float(scale), eps, dict(names)
         self.key_dim = kv_rank + rot_dim
-        if not 1 <= self.key_dim <= 256:
-            raise ValueError(f"latent_attention: a kept key of {self.key_dim} numbers; the attention kernels take up to 256")
+        self.head_width = max(head_dim + rot_dim, value_dim)      # "heads": keys and values padded with zeros to one width
+        if keep not in (None, "latent", "heads"):
+            raise ValueError(f"latent_attention: keep = {keep!r}")
+        self.keep = keep or ("latent" if self.key_dim <= 256 else "heads")
+        kept = self.key_dim if self.keep == "latent" else self.head_width
+        if not 1 <= kept <= 256:
+            raise ValueError(f"latent_attention: a kept key of {kept} numbers; the attention kernels take up to 256")
         self.q_width = n_heads * (head_dim + rot_dim)
         self.o_width = n_heads * value_dim
         # one product for everything that reads h: q | dkv | g
@@ -141,15 +149,17 @@ class LatentAttention(Part):
             ParamSpec(self.names["dkv_norm"], (r,), "vector", ("normal", 1.0, 0.1))]
 
     def cache_spec(self):
-        return PagedKV(1, self.key_dim)
+        return PagedKV(1, self.key_dim) if self.keep == "latent" else PagedKV(self.n_heads, self.head_width)
 
     def bind(self, tensors, runtime):
         super().bind(tensors, runtime)
         self.proj.bind(tensors), self.out.bind(tensors)
         self.position.bind(tensors, runtime)
+        self.no_freq = torch.empty(0, dtype=torch.float32, device=runtime.device)
         H, r = self.n_heads, self.kv_rank
         # W_uk per head, transposed once: [heads, kv_rank, dim], so that both per-head products are out = W[h] a
         self.uk_t = tensors[self.names["uk"]].view(H, self.head_dim, r).transpose(1, 2).contiguous()
+        self.uk = tensors[self.names["uk"]].view(H, self.head_dim, r).contiguous()
         self.uv = tensors[self.names["uv"]].view(H, self.value_dim, r).contiguous()
         self.c_norm = tensors[self.names["dkv_norm"]]
 
@@ -159,6 +169,8 @@ class LatentAttention(Part):
         g = ctx.groups[cache.group]
         z = self.proj(h, out_dtype=torch.float32)
         low, gate = self.q_width, self.q_width + kd
+        if self.keep == "heads":
+            return self._forward_heads(z, ctx, cache, g, accumulate_into)
         # the token's key: [c | turned part]
         key = torch.empty((T, kd), dtype=act, device=h.device)
         ops.rmsnorm(z[:, low:low + r], self.c_norm, self.eps, key[:, :r])
@@ -175,5 +187,34 @@ class LatentAttention(Part):
         o = torch.empty((T, self.o_width), dtype=torch.float32, device=h.device)
         ops.heads_linear(o_lat, self.uv, o, a_off=0, a_stride=kd)
         og = torch.empty((T, self.o_width), dtype=act, device=h.device)
+        ops.gated(o, z[:, gate:], "sigmoid", og)
+        self.out(og, residual=accumulate_into)
+
+    def _forward_heads(self, z, ctx, cache, g, accumulate_into):
+        """Every head's key [W_uk c | turned part | zeros] and value [W_uv c | zeros], `head_width` wide, go to the cache;
+        the queries are [q_plain | turned part | zeros]: the zeros add nothing to a score or a result."""
+        act, T, H, dev = self.runtime.act_dtype, z.shape[0], self.n_heads, z.device
+        dn, dr, r, dv, hw = self.head_dim, self.rot_dim, self.kv_rank, self.value_dim, self.head_width
+        low, gate = self.q_width, self.q_width + self.key_dim
+        copy = lambda src, dst, width, **layout: ops.rotary(src, dst, ctx.positions, self.no_freq, H, 0, width, **layout)   # noqa: E731
+        c = torch.empty((T, r), dtype=act, device=dev)
+        ops.rmsnorm(z[:, low:low + r], self.c_norm, self.eps, c)
+        kv = torch.zeros((T, 2 * H * hw), dtype=act, device=dev)      # keys at column 0, values at H * hw
+        ops.heads_linear(c, self.uk, kv, a_off=0, a_stride=0, o_off=0, o_stride=hw)
+        self.position.turn(z, kv, ctx.positions, H, dr, src_off=low + r, src_stride=0, dst_off=dn, dst_stride=hw)
+        ops.heads_linear(c, self.uv, kv, a_off=0, a_stride=0, o_off=H * hw, o_stride=hw)
+        if cache.writes:
+            ops.kv_write(kv, 0, H * hw, g.slot_map, cache.k, cache.v)
+        q = torch.zeros((T, H * hw), dtype=act, device=dev)
+        copy(z, q, dn, src_off=0, src_stride=dn + dr, dst_off=0, dst_stride=hw)
+        self.position.turn(z, q, ctx.positions, H, dr, src_off=dn, src_stride=dn + dr, dst_off=dn, dst_stride=hw)
+        o = torch.empty((T, H * hw), dtype=act, device=dev)
+        ops.attention(q, o, cache.k, cache.v, g.block_tables, g.tiles, H, self.scale, 0, tiles_wide=g.tiles_wide,
+                      single_rows=g.single_rows, max_context=g.max_context)
+        if hw != dv:
+            packed = torch.empty((T, self.o_width), dtype=act, device=dev)
+            copy(o, packed, dv, src_off=0, src_stride=hw, dst_off=0, dst_stride=dv)
+            o = packed
+        og = torch.empty((T, self.o_width), dtype=act, device=dev)
         ops.gated(o, z[:, gate:], "sigmoid", og)
         self.out(og, residual=accumulate_into)

@@ -382,7 +382,8 @@ def moe_plan(ids, n_experts, offsets, order):
     offsets[1:] = torch.cumsum(counts, 0).to(torch.int32)
 
 
-def moe_up(h, order, offsets, top, w_gate, w_up, limit, alpha, y):
+def moe_up(h, order, offsets, top, w_gate, w_up, limit, alpha, y, dims=None):
+    assert dims is None, "packed experts are for the GPU's kernels"
     off = offsets.tolist()
     for e in range(w_gate.shape[0]):
         for p in range(off[e], off[e + 1]):
@@ -392,7 +393,8 @@ def moe_up(h, order, offsets, top, w_gate, w_up, limit, alpha, y):
             y[p] = (g * torch.sigmoid(alpha * g) * (u + 1.0)).to(y.dtype)
 
 
-def moe_down(y, order, offsets, w_down, out):
+def moe_down(y, order, offsets, w_down, out, dims=None):
+    assert dims is None, "packed experts are for the GPU's kernels"
     off = offsets.tolist()
     for e in range(w_down.shape[0]):
         for p in range(off[e], off[e + 1]):

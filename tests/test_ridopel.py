@@ -17,10 +17,12 @@ from plain import ridopel_plain as plain
 # ----------------------------------------------------------------------------------------------------------------
 # configurations: none has the sizes of any model that is shipped anywhere; each differs from the others in every size
 # ----------------------------------------------------------------------------------------------------------------
-def latent(heads=2, dim=16, rot_dim=8, vdim=16, kv_rank=24, dims=None, base=10000.0, scale=None):
-    return dict(type="latent_attention", mixer=dict(heads=heads, dim=dim, rot_dim=rot_dim, vdim=vdim, kv_rank=kv_rank,
-                                                    scale=scale if scale is not None else (dim + rot_dim) ** -0.5,
-                                                    rot=dict(base=base, dims=rot_dim if dims is None else dims)))
+def latent(heads=2, dim=16, rot_dim=8, vdim=16, kv_rank=24, dims=None, base=10000.0, scale=None, keep=None):
+    m = dict(heads=heads, dim=dim, rot_dim=rot_dim, vdim=vdim, kv_rank=kv_rank,
+             scale=scale if scale is not None else (dim + rot_dim) ** -0.5, rot=dict(base=base, dims=rot_dim if dims is None else dims))
+    if keep:
+        m["keep"] = keep      # (what the cache holds: the latent, or every head's own keys and values)
+    return dict(type="latent_attention", mixer=m)
 
 
 def wkv(heads=2, dim=16, rank=8):
@@ -55,9 +57,10 @@ CFG_P = config([with_mlp(wkv(2, 16, 8), moe(24, 4, 2)), with_mlp(latent(2, 16, 8
                 with_mlp(hgrn2(2, 16, 8), None), with_mlp(latent(2, 16, 8, 16, 24), moe(24, 4, 2))],
                width=32, vocab=97, taps=3, loop=(1, 3, 2))
 # other sizes: one head, values wider than keys, fewer turned dimensions than rot_dim, a kept key that is no multiple of
-# 16 (40 + 12), four taps, one expert of three, all five experts, three passes over one layer, no soft cap
+# 16 (40 + 12), a latent attention that keeps every head's keys, four taps, one expert of three, all five experts, three
+# passes over one layer, no soft cap
 CFG_Q = config([with_mlp(hgrn2(3, 8, 24), moe(16, 3, 1, 1.5)), with_mlp(latent(1, 24, 12, 40, 40, dims=8, base=300.0), moe(40, 5, 5, 2.5)),
-                with_mlp(wkv(1, 40, 5), moe(16, 3, 1, 1.5)), with_mlp(latent(3, 8, 4, 8, 12, base=50000.0), None)],
+                with_mlp(wkv(1, 40, 5), moe(16, 3, 1, 1.5)), with_mlp(latent(3, 8, 4, 8, 12, base=50000.0, keep="heads"), None)],
                width=48, vocab=131, taps=4, loop=(0, 1, 3), eps=1e-6, softcap=0)
 # no loop, no convolution
 CFG_R = config([with_mlp(latent(4, 8, 8, 8, 8), moe(8, 2, 1)), with_mlp(wkv(4, 8, 4), moe(8, 2, 2))], width=32, vocab=61, taps=0)
@@ -146,6 +149,8 @@ def seqs_for(cfg, lengths, seed=3):
 ALONE = {
     "latent": [with_mlp(latent(3, 8, 8, 16, 16), None)],
     "latent_part_turned": [with_mlp(latent(2, 12, 12, 4, 20, dims=6), None)],
+    "latent_heads_kept": [with_mlp(latent(2, 12, 4, 24, 20, keep="heads"), None)],
+    "latent_heads_kept_narrow_values": [with_mlp(latent(3, 8, 8, 8, 16, dims=4, keep="heads"), None)],
     "wkv": [with_mlp(wkv(3, 8, 6), None)],
     "hgrn2": [with_mlp(hgrn2(2, 24, 8), None)],
     "experts": [with_mlp(hgrn2(1, 8, 8), moe(12, 6, 3, 0.7))],
