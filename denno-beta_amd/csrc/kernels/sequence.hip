@@ -201,9 +201,11 @@ __global__ __launch_bounds__(256) void gated_kernel(const void* x, int x_dt, siz
 // channels, 16 beyond), so a wave has 64 / KG columns and a column's parts are joined inside a row of 16 lanes,
 // without LDS; a part's sum over i runs in ascending order, one fused multiply-add a step, and the parts are joined
 // in one fixed order, whatever the step holds.
-// A row's r, k and w reach the lanes through LDS, eight rows at a time; the next eight are asked for before the
+// A row's r, k and w reach the lanes through LDS, some rows at a time (16, or 2 in a step of single rows); the next are asked for before the
 // current ones are worked on.  Places beyond a request's last row hold r = 0, a = 0, w = 1, which change nothing, so the
-// eight rows are worked on without a branch between them.
+// rows of a fetch are worked on without a branch between them.
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
+
 struct ScanArgs {
   const float *r, *k, *v, *w, *u;
   size_t ldr, ldk, ldv, ldw;
@@ -215,15 +217,19 @@ struct ScanArgs {
   size_t ldo;
 };
 
-template <int DK, int KG, bool AFTER>
+template <int DK, int KG, bool AFTER, bool VEC, int TB>
 __global__ __launch_bounds__(64) void scan_kernel(ScanArgs a) {
   constexpr int KQ = DK / KG;
+  constexpr int CW = 64 / KG;      // value columns of a wave
   constexpr int NL = DK >= 64 ? DK / 64 : 1;
-  constexpr int TB = 8;      // rows asked for at a time: a trip to memory is paid once per eight rows, not per row
+  // TB: rows asked for at a time (a trip to memory is paid once per TB rows, not per row; all TB places are worked on,
+  // so steps of single rows take a small TB).  A row's sums are the same for every TB.
+  constexpr int N4 = TB * DK / 4, NV = N4 >= 64 ? N4 / 64 : 1;      // VEC: groups of four numbers per array, per lane
   __shared__ __attribute__((aligned(16))) float sh[TB][3 * DK];
+  __shared__ __attribute__((aligned(16))) float shv[TB][CW];
   __shared__ __attribute__((aligned(16))) float shu[DK];
   const int s = blockIdx.z, h = blockIdx.y, lane = threadIdx.x;
-  const int kg = lane % KG, j = blockIdx.x * (64 / KG) + lane / KG;
+  const int kg = lane % KG, j0 = blockIdx.x * CW, j = j0 + lane / KG;
   const int slot = a.slots[s];
   if (slot < 0) return;
   const int row0 = a.row_start[s], row1 = a.row_start[s + 1];
@@ -236,53 +242,89 @@ __global__ __launch_bounds__(64) void scan_kernel(ScanArgs a) {
 #pragma unroll
   for (int q = 0; q < KQ; ++q) S[q] = (live && kg * KQ + q < dk) ? sp[q] : 0.f;
   for (int i = lane; i < DK; i += 64) shu[i] = (a.u && i < dk) ? a.u[h * dk + i] : 0.f;
-  float nr[TB][NL], nk[TB][NL], nw[TB][NL], nv[TB];
+  // what a fetch brings: (not VEC) a lane's own numbers row by row; (VEC: every size a multiple of 4 and every row at a
+  // multiple of 16 bytes) 16 bytes a lane and load, eight rows of r, k or w in DK / 32 loads: a row then costs a wave
+  // 7 / 8 of a vector load where it cost four, and those loads, not the arithmetic, were what a row waited for
+  float nr[VEC ? 1 : TB][NL], nk[VEC ? 1 : TB][NL], nw[VEC ? 1 : TB][NL], nv[VEC ? 1 : TB];
+  f32x4 r4[VEC ? NV : 1], k4[VEC ? NV : 1], w4[VEC ? NV : 1], v4;
   auto fetch = [&](int t0) {
+    if constexpr (VEC) {
+      const f32x4 zero = {0.f, 0.f, 0.f, 0.f}, one = {1.f, 1.f, 1.f, 1.f};
 #pragma unroll
-    for (int b = 0; b < TB; ++b) {
-      const int t = t0 + b;
-      const bool row = t < row1;
-#pragma unroll
-      for (int q = 0; q < NL; ++q) {
-        const int i = lane + 64 * q;
-        const bool ok = row && i < dk;
-        nr[b][q] = ok ? a.r[t * a.ldr + h * dk + i] : 0.f;
-        nk[b][q] = (ok && !a.key_from_decay) ? a.k[t * a.ldk + h * dk + i] : 0.f;
-        nw[b][q] = ok ? a.w[t * a.ldw + h * dk + i] : 1.f;
+      for (int it = 0; it < NV; ++it) {
+        const int idx = it * 64 + lane, bq = idx / (DK / 4), i = (idx % (DK / 4)) * 4, t = t0 + bq;
+        const bool ok = idx < N4 && t < row1 && i < dk;
+        r4[it] = ok ? *reinterpret_cast<const f32x4*>(a.r + t * a.ldr + h * dk + i) : zero;
+        k4[it] = (ok && !a.key_from_decay) ? *reinterpret_cast<const f32x4*>(a.k + t * a.ldk + h * dk + i) : zero;
+        w4[it] = ok ? *reinterpret_cast<const f32x4*>(a.w + t * a.ldw + h * dk + i) : one;
       }
-      nv[b] = (row && live) ? a.v[t * a.ldv + h * dv + j] : 0.f;
+      const int bq = lane / (CW / 4), col = j0 + (lane % (CW / 4)) * 4, t = t0 + bq;
+      v4 = (lane < TB * CW / 4 && t < row1 && col < dv) ? *reinterpret_cast<const f32x4*>(a.v + t * a.ldv + h * dv + col) : zero;
+    } else {
+#pragma unroll
+      for (int bq = 0; bq < TB; ++bq) {
+        const int t = t0 + bq;
+        const bool row = t < row1;
+#pragma unroll
+        for (int q = 0; q < NL; ++q) {
+          const int i = lane + 64 * q;
+          const bool ok = row && i < dk;
+          nr[bq][q] = ok ? a.r[t * a.ldr + h * dk + i] : 0.f;
+          nk[bq][q] = (ok && !a.key_from_decay) ? a.k[t * a.ldk + h * dk + i] : 0.f;
+          nw[bq][q] = ok ? a.w[t * a.ldw + h * dk + i] : 1.f;
+        }
+        nv[bq] = (row && live) ? a.v[t * a.ldv + h * dv + j] : 0.f;
+      }
     }
   };
   fetch(row0);
   for (int t0 = row0; t0 < row1; t0 += TB) {
     float vj[TB];
+    if constexpr (VEC) {
 #pragma unroll
-    for (int b = 0; b < TB; ++b) {
-#pragma unroll
-      for (int q = 0; q < NL; ++q) {
-        const int i = lane + 64 * q;
-        if (i < DK) {
-          sh[b][i] = nr[b][q];
-          sh[b][DK + i] = a.key_from_decay ? 1.0f - nw[b][q] : nk[b][q];
-          sh[b][2 * DK + i] = nw[b][q];
+      for (int it = 0; it < NV; ++it) {
+        const int idx = it * 64 + lane, bq = idx / (DK / 4), i = (idx % (DK / 4)) * 4;
+        if (idx < N4) {
+          const f32x4 one = {1.f, 1.f, 1.f, 1.f};
+          *reinterpret_cast<f32x4*>(&sh[bq][i]) = r4[it];
+          *reinterpret_cast<f32x4*>(&sh[bq][DK + i]) = a.key_from_decay ? one - w4[it] : k4[it];
+          *reinterpret_cast<f32x4*>(&sh[bq][2 * DK + i]) = w4[it];
         }
       }
-      vj[b] = nv[b];
+      if (lane < TB * CW / 4) *reinterpret_cast<f32x4*>(&shv[lane / (CW / 4)][(lane % (CW / 4)) * 4]) = v4;
+    } else {
+#pragma unroll
+      for (int bq = 0; bq < TB; ++bq) {
+#pragma unroll
+        for (int q = 0; q < NL; ++q) {
+          const int i = lane + 64 * q;
+          if (i < DK) {
+            sh[bq][i] = nr[bq][q];
+            sh[bq][DK + i] = a.key_from_decay ? 1.0f - nw[bq][q] : nk[bq][q];
+            sh[bq][2 * DK + i] = nw[bq][q];
+          }
+        }
+        vj[bq] = nv[bq];
+      }
     }
     __syncthreads();
+    if constexpr (VEC) {
+#pragma unroll
+      for (int bq = 0; bq < TB; ++bq) vj[bq] = shv[bq][lane / KG];
+    }
     if (t0 + TB < row1) fetch(t0 + TB);
     // (no branch inside the eight rows: their reads, sums and joins can then overlap)
     float ob[TB];
 #pragma unroll
-    for (int b = 0; b < TB; ++b) {
-      const float* mr = sh[b] + kg * KQ;
+    for (int bq = 0; bq < TB; ++bq) {
+      const float* mr = sh[bq] + kg * KQ;
       const float* mk = mr + DK;
       const float* mw = mk + DK;
       const float* mu = shu + kg * KQ;
       float o = 0.f;
 #pragma unroll
       for (int q = 0; q < KQ; ++q) {
-        const float kv = mk[q] * vj[b];
+        const float kv = mk[q] * vj[bq];
         if (AFTER) {
           S[q] = fmaf(mw[q], S[q], kv);
           o = fmaf(mr[q], S[q], o);
@@ -291,12 +333,12 @@ __global__ __launch_bounds__(64) void scan_kernel(ScanArgs a) {
           S[q] = fmaf(mw[q], S[q], kv);
         }
       }
-      ob[b] = group_reduce<KG>(o, SumOp());
+      ob[bq] = group_reduce<KG>(o, SumOp());
     }
     if (live && kg == 0) {
 #pragma unroll
-      for (int b = 0; b < TB; ++b)
-        if (t0 + b < row1) a.out[(t0 + b) * a.ldo + h * dv + j] = ob[b];
+      for (int bq = 0; bq < TB; ++bq)
+        if (t0 + bq < row1) a.out[(t0 + bq) * a.ldo + h * dv + j] = ob[bq];
     }
     __syncthreads();
   }
@@ -412,7 +454,7 @@ int dn_gated(const void* x, int x_dt, long long ldx, const float* g, long long l
 
 int dn_state_scan(const float* r, long long ldr, const float* k, long long ldk, const float* v, long long ldv, const float* w,
                   long long ldw, const float* u, float* state, long long slot_stride, const int* row_start, const int* slots, int S,
-                  int H, int dk, int dv, int read_after, int key_from_decay, float* out, long long ldo, hipStream_t stream) {
+                  int T, int H, int dk, int dv, int read_after, int key_from_decay, float* out, long long ldo, hipStream_t stream) {
   if (dk < 1 || dk > 256 || dv < 1 || H < 1) return DN_ERR_SHAPE;
   if (!key_from_decay && k == nullptr) return DN_ERR_SHAPE;
   if (S == 0) return 0;
@@ -421,16 +463,32 @@ int dn_state_scan(const float* r, long long ldr, const float* k, long long ldk, 
              static_cast<size_t>(ldo)};
   // (the parts of a column's sum by the head's size alone, never by the step: a row's bits are the same in every step)
   const dim3 few((dv + 15) / 16, H, S), many((dv + 3) / 4, H, S);
-#define DN_SCAN(DK, KG, GRID)                                                                       \
-  do {                                                                                             \
-    if (read_after) hipLaunchKernelGGL((scan_kernel<DK, KG, true>), GRID, dim3(64), 0, stream, a); \
-    else hipLaunchKernelGGL((scan_kernel<DK, KG, false>), GRID, dim3(64), 0, stream, a);           \
+  auto by16 = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
+  const bool vec = dk % 4 == 0 && dv % 4 == 0 && ldr % 4 == 0 && ldv % 4 == 0 && ldw % 4 == 0 && (key_from_decay || ldk % 4 == 0) &&
+                   by16(r) && by16(v) && by16(w) && (key_from_decay || by16(k));
+  const bool few_rows = T <= 2 * S;      // (decoded tokens: a row or two a request)
+#define DN_SCAN3(DK, KG, GRID, AFTER, VEC)                                                                    \
+  do {                                                                                                        \
+    if (few_rows) hipLaunchKernelGGL((scan_kernel<DK, KG, AFTER, VEC, 2>), GRID, dim3(64), 0, stream, a);  \
+    else hipLaunchKernelGGL((scan_kernel<DK, KG, AFTER, VEC, (VEC ? 16 : 8)>), GRID, dim3(64), 0, stream, a); \
+  } while (0)
+#define DN_SCAN2(DK, KG, GRID, AFTER)        \
+  do {                                       \
+    if (vec) DN_SCAN3(DK, KG, GRID, AFTER, true); \
+    else DN_SCAN3(DK, KG, GRID, AFTER, false);    \
+  } while (0)
+#define DN_SCAN(DK, KG, GRID)                \
+  do {                                       \
+    if (read_after) DN_SCAN2(DK, KG, GRID, true); \
+    else DN_SCAN2(DK, KG, GRID, false);      \
   } while (0)
   if (dk <= 16) DN_SCAN(16, 4, few);
   else if (dk <= 32) DN_SCAN(32, 4, few);
   else if (dk <= 64) DN_SCAN(64, 16, many);
   else if (dk <= 128) DN_SCAN(128, 16, many);
   else DN_SCAN(256, 16, many);
+#undef DN_SCAN2
+#undef DN_SCAN3
 #undef DN_SCAN
   return dn_launch_status();
 }

@@ -131,7 +131,7 @@ def _declare(name, lib):
             "dn_rotary": [P, I, c_longlong, I, I, P, I, c_longlong, I, I, P, P, I, I, I, I, P],
             "dn_activate": [P, c_longlong, P, P, I, P, I, c_longlong, I, I, P],
             "dn_gated": [P, I, c_longlong, P, c_longlong, I, P, I, c_longlong, I, I, P],
-            "dn_state_scan": [P, c_longlong, P, c_longlong, P, c_longlong, P, c_longlong, P, P, c_longlong, P, P, I, I, I, I, I, I,
+            "dn_state_scan": [P, c_longlong, P, c_longlong, P, c_longlong, P, c_longlong, P, P, c_longlong, P, P, I, I, I, I, I, I, I,
                               P, c_longlong, P],
             "dn_head_norm": [P, c_longlong, P, I, F, P, c_longlong, I, P, I, c_longlong, I, I, I, P],
         },
@@ -1067,7 +1067,7 @@ def state_scan(r, k, v, w, u, state, row_start, slots, n_heads, dk, dv, out, rea
     _ok(_lib("sequence").dn_state_scan(r.data_ptr(), _rows(r, "r"), 0 if key_from_decay else k.data_ptr(),
                                        0 if key_from_decay else _rows(k, "k"), v.data_ptr(), _rows(v, "v"), w.data_ptr(),
                                        _rows(w, "w"), _ptr(u), state.data_ptr(), stride, row_start.data_ptr(), slots.data_ptr(), S,
-                                       n_heads, dk, dv, int(read_after), int(key_from_decay), out.data_ptr(), _rows(out, "out"),
+                                       T, n_heads, dk, dv, int(read_after), int(key_from_decay), out.data_ptr(), _rows(out, "out"),
                                        _stream()), "state_scan")
     return out
 

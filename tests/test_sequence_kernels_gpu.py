@@ -95,10 +95,13 @@ def test_activate_and_gated(kind):
         both("gated", lambda: (x.bfloat16(), g, kind, torch.empty(6, 45, dtype=torch.bfloat16, device=DEV)), [3], torch.bfloat16)
 
 
-@pytest.mark.parametrize("dk,dv,heads", [(16, 16, 2), (48, 32, 3), (5, 70, 1), (64, 64, 4), (100, 9, 2), (130, 20, 1)])
+# (sizes that are multiples of 4 take the fetches of 16 bytes a lane, the others the fetches of single numbers)
+@pytest.mark.parametrize("dk,dv,heads", [(16, 16, 2), (48, 32, 3), (5, 70, 1), (64, 64, 4), (100, 9, 2), (130, 20, 1), (32, 12, 2),
+                                         (128, 36, 1), (252, 8, 1), (64, 128, 2)])
 @pytest.mark.parametrize("mode", ["bonus", "gate"])
-def test_state_scan(dk, dv, heads, mode):
-    row_start, slots, T = tables([1, 12, 3], [2, -1, 0])
+@pytest.mark.parametrize("lengths", [[1, 12, 40], [1, 2, 1]])      # portions; a step of single rows (another kernel variant)
+def test_state_scan(dk, dv, heads, mode, lengths):
+    row_start, slots, T = tables(lengths, [2, -1, 0])
     r, k = torch.randn(T, heads * dk, device=DEV), torch.randn(T, heads * dk, device=DEV)
     v = torch.randn(T, heads * dv, device=DEV)
     w = torch.rand(T, heads * dk, device=DEV) * 0.5 + 0.5
