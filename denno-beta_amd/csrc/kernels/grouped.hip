@@ -115,6 +115,45 @@ __global__ __launch_bounds__(64) void route_kernel(const float* z, const float* 
   for (int c = 0; c < top; ++c) wts[t * top + c] *= inv;
 }
 
+// The same choice with a wave a row (up to 8,192 experts, `top` up to 64): lane l has the experts l, l + 64, ...; the
+// largest score is found over the lanes, the lowest index among equals wins, and lane c keeps the c-th choice.
+__global__ __launch_bounds__(64) void route_wave_kernel(const float* z, const float* correction, int E, int top, int* ids, float* wts) {
+  const int t = blockIdx.x, lane = threadIdx.x;
+  const float* row = z + static_cast<size_t>(t) * E;
+  const float none = -__builtin_huge_valf();
+  float m = none;
+  for (int e = lane; e < E; e += 64) m = fmaxf(m, row[e]);
+  m = wave_max(m);
+  float sum = 0.f;
+  for (int e = lane; e < E; e += 64) sum += expf(row[e] - m);
+  sum = wave_sum(sum);
+  unsigned taken[4] = {0u, 0u, 0u, 0u};      // a bit for each of the lane's up to 128 experts
+  float my_w = 0.f;
+  int my_id = 0;
+  for (int c = 0; c < top; ++c) {
+    float best_v = none, best_s = 0.f;
+    int best = 0x7fffffff;
+    for (int e = lane, k = 0; e < E; e += 64, ++k) {
+      if ((taken[k >> 5] >> (k & 31)) & 1u) continue;
+      const float sc = expf(row[e] - m) / sum;
+      const float v = sc + (correction ? correction[e] : 0.f);
+      if (v > best_v) best_v = v, best = e, best_s = sc;
+    }
+    const float top_v = wave_max(best_v);
+    int win = static_cast<int>(-wave_max(-static_cast<float>((best_v == top_v && best < E) ? best : 16777216)));
+    if (win >= E) win = c;      // (scores that are no numbers: any expert, never an index outside)
+    const bool mine = (win & 63) == lane;
+    const float s_win = wave_max((mine && best == win) ? best_s : none);
+    if (mine) taken[(win >> 6) >> 5] |= 1u << ((win >> 6) & 31);
+    if (lane == c) my_id = win, my_w = s_win > none ? s_win : 0.f;
+  }
+  const float chosen = wave_sum(lane < top ? my_w : 0.f);
+  if (lane < top) {
+    ids[t * top + lane] = my_id;
+    wts[t * top + lane] = my_w / (chosen + 1e-20f);
+  }
+}
+
 // ---- the plan ------------------------------------------------------------------------------------------------
 // The n pairs (row, choice), pair i = row * top + choice, sorted by expert and inside an expert by i:
 // offsets[e] .. offsets[e + 1] - 1 are expert e's places in `order`.  One workgroup.
@@ -416,34 +455,37 @@ __global__ __launch_bounds__(256) void expert_down_mfma_kernel(const bf16_t* y, 
 
 
 // The same two kernels for packed weights (the experts' matrices stacked and packed as one; an expert's rows start at a
-// multiple of 16): a wave takes 32 pairs x 64 columns, a workgroup 64 x 128.
+// multiple of 16): a wave takes 32 pairs x 64 columns, a workgroup 64 x 128; where the step has few pairs an expert
+// (decoded tokens: the kernel then only streams the chosen experts' matrices) a wave takes 16 columns, so that four
+// times as many waves have loads in flight.  An element's sum is the same in both.
+template <int CB>
 __global__ __launch_bounds__(256) void expert_up_packed_kernel(const bf16_t* h, size_t ldh, const int* order, const int* offsets, int E,
                                                                int top, const bf16_t* wg, const bf16_t* wu, int ff, int width,
                                                                float limit, float alpha, bf16_t* y, int tiles_x) {
   int e, p0, p1, tx, ty;
-  xcd_tile(tiles_x, (ff + 127) / 128, tx, ty);
+  xcd_tile(tiles_x, (ff + 32 * CB - 1) / (32 * CB), tx, ty);
   if (tx < 0 || !expert_tile64(offsets, E, tx, e, p0, p1)) return;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int pw = p0 + (wave >> 1) * 32, nw = ty * 128 + (wave & 1) * 64;
+  const int pw = p0 + (wave >> 1) * 32, nw = ty * (32 * CB) + (wave & 1) * (16 * CB);
   if (pw >= p1 || nw >= ff) return;
   const int kq = (lane >> 4) * 8, lr = lane & 15, ksteps = width / 32;
-  const bf16_t *a_ptr[2], *g_ptr[4], *u_ptr[4];
+  const bf16_t *a_ptr[2], *g_ptr[CB], *u_ptr[CB];
 #pragma unroll
   for (int i = 0; i < 2; ++i) a_ptr[i] = h + static_cast<size_t>(order[min(pw + 16 * i + lr, p1 - 1)] / top) * ldh + kq;
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
+  for (int j = 0; j < CB; ++j) {
     const size_t block = (static_cast<size_t>(e) * ff + min(nw + 16 * j, ff - 16)) / 16;
     g_ptr[j] = wg + block * ksteps * 512 + lane * 8;
     u_ptr[j] = wu + block * ksteps * 512 + lane * 8;
   }
-  f32x4 g[2][4] = {}, u[2][4] = {};
-  mfma_tile<true, true, 4>(a_ptr, g_ptr, u_ptr, width, g, u);
+  f32x4 g[2][CB] = {}, u[2][CB] = {};
+  mfma_tile<true, true, CB>(a_ptr, g_ptr, u_ptr, width, g, u);
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
     const int p = pw + 16 * i + lr;
     if (p >= p1) continue;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < CB; ++j) {
       const int n = nw + 16 * j + (lane >> 4) * 4;
       if (n >= ff) continue;      // (ff is a multiple of 16: a block is whole or absent)
 #pragma unroll
@@ -455,30 +497,31 @@ __global__ __launch_bounds__(256) void expert_up_packed_kernel(const bf16_t* h, 
   }
 }
 
+template <int CB>
 __global__ __launch_bounds__(256) void expert_down_packed_kernel(const bf16_t* y, const int* order, const int* offsets, int E,
                                                                  const bf16_t* wd, int width, int ff, float* out, int tiles_x) {
   int e, p0, p1, tx, ty;
-  xcd_tile(tiles_x, (width + 127) / 128, tx, ty);
+  xcd_tile(tiles_x, (width + 32 * CB - 1) / (32 * CB), tx, ty);
   if (tx < 0 || !expert_tile64(offsets, E, tx, e, p0, p1)) return;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int pw = p0 + (wave >> 1) * 32, nw = ty * 128 + (wave & 1) * 64;
+  const int pw = p0 + (wave >> 1) * 32, nw = ty * (32 * CB) + (wave & 1) * (16 * CB);
   if (pw >= p1 || nw >= width) return;
   const int kq = (lane >> 4) * 8, lr = lane & 15, ksteps = ff / 32;
-  const bf16_t *a_ptr[2], *w_ptr[4];
+  const bf16_t *a_ptr[2], *w_ptr[CB];
 #pragma unroll
   for (int i = 0; i < 2; ++i) a_ptr[i] = y + static_cast<size_t>(min(pw + 16 * i + lr, p1 - 1)) * ff + kq;
 #pragma unroll
-  for (int j = 0; j < 4; ++j)
+  for (int j = 0; j < CB; ++j)
     w_ptr[j] = wd + (static_cast<size_t>(e) * width + min(nw + 16 * j, width - 16)) / 16 * ksteps * 512 + lane * 8;
-  f32x4 acc[2][4] = {};
-  mfma_tile<false, true, 4>(a_ptr, w_ptr, nullptr, ff, acc, nullptr);
+  f32x4 acc[2][CB] = {};
+  mfma_tile<false, true, CB>(a_ptr, w_ptr, nullptr, ff, acc, nullptr);
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
     const int p = pw + 16 * i + lr;
     if (p >= p1) continue;
     const size_t pair = order[p];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < CB; ++j) {
       const int n = nw + 16 * j + (lane >> 4) * 4;
       if (n >= width) continue;
       *reinterpret_cast<f32x4*>(out + pair * width + n) = acc[i][j];
@@ -544,6 +587,10 @@ int dn_heads_linear(const void* a, int a_dt, long long lda, int a_off, int a_str
 int dn_moe_route(const float* z, const float* correction, int T, int E, int top, int* ids, float* wts, hipStream_t stream) {
   if (E < 1 || top < 1 || top > E) return DN_ERR_SHAPE;
   if (T == 0) return 0;
+  if (E <= 8192 && top <= 64) {
+    hipLaunchKernelGGL(route_wave_kernel, dim3(T), dim3(64), 0, stream, z, correction, E, top, ids, wts);
+    return dn_launch_status();
+  }
   hipLaunchKernelGGL(route_kernel, dim3((T + 63) / 64), dim3(64), 0, stream, z, correction, T, E, top, ids, wts);
   return dn_launch_status();
 }
@@ -565,10 +612,18 @@ int dn_moe_up(const void* h, int h_dt, long long ldh, const int* order, const in
   if (packed) {
     if (h_dt != DN_BF16 || w_dt != DN_BF16 || y_dt != DN_BF16) return DN_ERR_DTYPE;
     if (width % 32 != 0 || ff % 16 != 0 || ldh % 8 != 0 || !aligned16(h) || !aligned16(wg) || !aligned16(wu)) return DN_ERR_SHAPE;
-    const int tiles_x = (n + MT - 1) / MT + E, tiles = tiles_x * ((ff + 127) / 128);
-    hipLaunchKernelGGL(expert_up_packed_kernel, dim3((tiles + 7) / 8 * 8), dim3(256), 0, stream, static_cast<const bf16_t*>(h),
-                       static_cast<size_t>(ldh), order, offsets, E, top, static_cast<const bf16_t*>(wg), static_cast<const bf16_t*>(wu),
-                       ff, width, limit, alpha, static_cast<bf16_t*>(y), tiles_x);
+    const int tiles_x = (n + MT - 1) / MT + E;
+    if (n <= 16 * E) {
+      const int tiles = tiles_x * ((ff + 31) / 32);
+      hipLaunchKernelGGL(expert_up_packed_kernel<1>, dim3((tiles + 7) / 8 * 8), dim3(256), 0, stream, static_cast<const bf16_t*>(h),
+                         static_cast<size_t>(ldh), order, offsets, E, top, static_cast<const bf16_t*>(wg),
+                         static_cast<const bf16_t*>(wu), ff, width, limit, alpha, static_cast<bf16_t*>(y), tiles_x);
+    } else {
+      const int tiles = tiles_x * ((ff + 127) / 128);
+      hipLaunchKernelGGL(expert_up_packed_kernel<4>, dim3((tiles + 7) / 8 * 8), dim3(256), 0, stream, static_cast<const bf16_t*>(h),
+                         static_cast<size_t>(ldh), order, offsets, E, top, static_cast<const bf16_t*>(wg),
+                         static_cast<const bf16_t*>(wu), ff, width, limit, alpha, static_cast<bf16_t*>(y), tiles_x);
+    }
     return dn_launch_status();
   }
   if (h_dt == DN_BF16 && w_dt == DN_BF16 && y_dt == DN_BF16 && width % 32 == 0 && ldh % 8 == 0 && aligned16(h) && aligned16(wg) &&
@@ -591,9 +646,16 @@ int dn_moe_down(const void* y, int y_dt, const int* order, const int* offsets, i
   if (packed) {
     if (y_dt != DN_BF16 || w_dt != DN_BF16) return DN_ERR_DTYPE;
     if (ff % 32 != 0 || width % 16 != 0 || !aligned16(y) || !aligned16(wd) || !aligned16(out)) return DN_ERR_SHAPE;
-    const int tiles_x = (n + MT - 1) / MT + E, tiles = tiles_x * ((width + 127) / 128);
-    hipLaunchKernelGGL(expert_down_packed_kernel, dim3((tiles + 7) / 8 * 8), dim3(256), 0, stream, static_cast<const bf16_t*>(y),
-                       order, offsets, E, static_cast<const bf16_t*>(wd), width, ff, out, tiles_x);
+    const int tiles_x = (n + MT - 1) / MT + E;
+    if (n <= 16 * E) {
+      const int tiles = tiles_x * ((width + 31) / 32);
+      hipLaunchKernelGGL(expert_down_packed_kernel<1>, dim3((tiles + 7) / 8 * 8), dim3(256), 0, stream, static_cast<const bf16_t*>(y),
+                         order, offsets, E, static_cast<const bf16_t*>(wd), width, ff, out, tiles_x);
+    } else {
+      const int tiles = tiles_x * ((width + 127) / 128);
+      hipLaunchKernelGGL(expert_down_packed_kernel<4>, dim3((tiles + 7) / 8 * 8), dim3(256), 0, stream, static_cast<const bf16_t*>(y),
+                         order, offsets, E, static_cast<const bf16_t*>(wd), width, ff, out, tiles_x);
+    }
     return dn_launch_status();
   }
   if (y_dt == DN_BF16 && w_dt == DN_BF16 && ff % 32 == 0 && aligned16(y) && aligned16(wd)) {

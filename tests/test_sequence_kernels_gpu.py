@@ -134,7 +134,7 @@ def test_heads_linear(dtype, T, H, N, K):
     both("heads_linear", lambda: (a, w, torch.zeros(T, 2 + H * (N + 1), dtype=dtype, device=DEV), 4, K + 3, 2, N + 1), [2], dtype)
 
 
-@pytest.mark.parametrize("T,E,top", [(1, 4, 2), (50, 16, 3), (700, 5, 5), (33, 70, 1)])
+@pytest.mark.parametrize("T,E,top", [(1, 4, 2), (50, 16, 3), (700, 5, 5), (33, 70, 1), (20, 200, 64), (7, 130, 70), (5, 64, 64)])
 def test_route_and_plan(T, E, top):
     z = torch.randn(T, E, device=DEV) * 2
     corr = torch.randn(E, device=DEV) * 0.1
