@@ -267,7 +267,7 @@ def ridopel_configs(width, layers=4, vocab=32000, positions=2048):
     H = width // 128
     moe = dict(kind="moe", expert=dict(ff=width, limit=7.0), router=dict(experts=16, top=2))
     lat = dict(type="latent_attention", mlp=moe, mixer=dict(heads=H, dim=64, rot_dim=32, vdim=128, kv_rank=224, scale=96 ** -0.5,
-                                                            rot=dict(base=500000.0, dims=32)))
+                                                            rot=dict(base=10000.0, dims=32)))
     kinds = [lat, dict(type="hgrn2", mlp=moe, mixer=dict(heads=H, dim=64, vdim=128)), lat,
              dict(type="wkv", mlp=moe, mixer=dict(heads=width // 64, dim=64, decay_rank=64))]
     rid = dict(architecture="Ridopel", vocab=vocab, width=width, norm=dict(eps=1e-5), canon=dict(taps=4), logit_softcap=30.0,
