@@ -199,14 +199,16 @@ __global__ __launch_bounds__(256) void plan_kernel(const int* ids, int n, int E,
 __global__ __launch_bounds__(256) void plan_runs_kernel(const int* ids, int n, int E, int* offsets, int* order) {
   extern __shared__ int cnt[];      // [256][E]
   const int tid = threadIdx.x;
-  const int L = (n + 255) / 256, lo = min(tid * L, n), hi = min(lo + L, n);
-  for (int e = 0; e < E; ++e) cnt[tid * E + e] = 0;
+  const int R = min(256, (n + 3) / 4);      // runs: four pairs a thread at least, so that few pairs make a short scan
+  const int L = (n + R - 1) / R, lo = min(tid * L, n), hi = min(lo + L, n);
+  if (tid < R)
+    for (int e = 0; e < E; ++e) cnt[tid * E + e] = 0;
   for (int i = lo; i < hi; ++i) cnt[tid * E + ids[i]] += 1;
   __syncthreads();
   __shared__ int total[49];
   if (tid < E) {
     int run = 0;
-    for (int t = 0; t < 256; ++t) {
+    for (int t = 0; t < R; ++t) {
       const int c = cnt[t * E + tid];
       cnt[t * E + tid] = run;
       run += c;
@@ -529,22 +531,45 @@ __global__ __launch_bounds__(256) void expert_down_packed_kernel(const bf16_t* y
   }
 }
 
-// out[t, o_off + h * o_stride + n] = sum_k W[h][n][k] a[t, a_off + h * a_stride + k], bfloat16 in, 32-bit sums
-__global__ __launch_bounds__(256) void heads_linear_mfma_kernel(const bf16_t* A, size_t lda, int a_off, int a_stride, const bf16_t* W,
+// out[t, o_off + h * o_stride + n] = sum_k W[h][n][k] a[t, a_off + h * a_stride + k] on the matrix cores, 32-bit sums.
+// AF32: the rows are 32-bit and are rounded to bfloat16 on their way into the instruction (two loads of 16 bytes a lane
+// and step in place of one).
+template <bool AF32>
+__global__ __launch_bounds__(256) void heads_linear_mfma_kernel(const void* A, size_t lda, int a_off, int a_stride, const bf16_t* W,
                                                                 void* out, int out_dt, size_t ldo, int o_off, int o_stride, int T,
                                                                 int N, int K) {
   const int hd = blockIdx.z, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int tw = blockIdx.x * MT + (wave >> 1) * 32, nw = blockIdx.y * 64 + (wave & 1) * 32;
   if (tw >= T || nw >= N) return;
   const int kq = (lane >> 4) * 8, lr = lane & 15;
-  const bf16_t *a_ptr[2], *w_ptr[2];
+  size_t a_at[2];
+  const bf16_t* w_ptr[2];
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
-    a_ptr[i] = A + static_cast<size_t>(min(tw + 16 * i + lr, T - 1)) * lda + a_off + static_cast<size_t>(hd) * a_stride + kq;
+    a_at[i] = static_cast<size_t>(min(tw + 16 * i + lr, T - 1)) * lda + a_off + static_cast<size_t>(hd) * a_stride + kq;
     w_ptr[i] = W + (static_cast<size_t>(hd) * N + min(nw + 16 * i + lr, N - 1)) * K + kq;
   }
   f32x4 acc[2][2] = {};
-  mfma_tile<false, false, 2>(a_ptr, w_ptr, nullptr, K, acc, nullptr);
+#pragma unroll 2
+  for (int k0 = 0; k0 < K; k0 += 32) {
+    bf16x8 af[2], wf[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      if constexpr (AF32) {
+        const float* p = static_cast<const float*>(A) + a_at[i] + k0;
+        const f32x4 lo = *reinterpret_cast<const f32x4*>(p), hi = *reinterpret_cast<const f32x4*>(p + 4);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) af[i][e] = static_cast<__bf16>(lo[e]), af[i][4 + e] = static_cast<__bf16>(hi[e]);
+      } else {
+        af[i] = load8(static_cast<const bf16_t*>(A) + a_at[i] + k0);
+      }
+      wf[i] = load8(w_ptr[i] + k0);
+    }
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[j], af[i], acc[i][j], 0, 0, 0);
+  }
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
     const int t = tw + 16 * i + lr;
@@ -572,11 +597,18 @@ int dn_heads_linear(const void* a, int a_dt, long long lda, int a_off, int a_str
   if (!float_kind(a_dt) || !float_kind(w_dt) || !float_kind(out_dt)) return DN_ERR_DTYPE;
   if (H < 1 || N < 1 || K < 1 || H > 65535) return DN_ERR_SHAPE;
   if (T == 0) return 0;
-  if (a_dt == DN_BF16 && w_dt == DN_BF16 && K % 32 == 0 && lda % 8 == 0 && a_off % 8 == 0 && a_stride % 8 == 0 && aligned16(a) &&
-      aligned16(w)) {
-    hipLaunchKernelGGL(heads_linear_mfma_kernel, dim3((T + MT - 1) / MT, (N + 63) / 64, H), dim3(256), 0, stream,
-                       static_cast<const bf16_t*>(a), static_cast<size_t>(lda), a_off, a_stride, static_cast<const bf16_t*>(w), out,
-                       out_dt, static_cast<size_t>(ldo), o_off, o_stride, T, N, K);
+  // bfloat16 weights take the matrix cores; 32-bit rows are rounded to bfloat16 on the way in, but only where the result
+  // is bfloat16 too (a 32-bit result of 32-bit rows keeps the vector kernel's 32-bit products)
+  const int per16 = a_dt == DN_BF16 ? 8 : 4;
+  if (w_dt == DN_BF16 && (a_dt == DN_BF16 || out_dt == DN_BF16) && K % 32 == 0 && lda % per16 == 0 && a_off % per16 == 0 &&
+      a_stride % per16 == 0 && aligned16(a) && aligned16(w)) {
+    const dim3 grid((T + MT - 1) / MT, (N + 63) / 64, H);
+    if (a_dt == DN_BF16)
+      hipLaunchKernelGGL(heads_linear_mfma_kernel<false>, grid, dim3(256), 0, stream, a, static_cast<size_t>(lda), a_off, a_stride,
+                         static_cast<const bf16_t*>(w), out, out_dt, static_cast<size_t>(ldo), o_off, o_stride, T, N, K);
+    else
+      hipLaunchKernelGGL(heads_linear_mfma_kernel<true>, grid, dim3(256), 0, stream, a, static_cast<size_t>(lda), a_off, a_stride,
+                         static_cast<const bf16_t*>(w), out, out_dt, static_cast<size_t>(ldo), o_off, o_stride, T, N, K);
     return dn_launch_status();
   }
   hipLaunchKernelGGL(heads_linear_kernel, dim3((T + TM - 1) / TM, (N + TN - 1) / TN, H), dim3(256), 0, stream, a, a_dt,

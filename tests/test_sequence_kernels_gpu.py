@@ -197,6 +197,9 @@ def test_heads_linear_on_the_matrix_cores(T, H, N, K):
     w = (torch.randn(H, N, K, device=DEV) / K ** 0.5).bfloat16()
     for dtype in DT:
         both("heads_linear", lambda: (a, w, torch.zeros(T, 2 + H * (N + 1), dtype=dtype, device=DEV), 8, K + 8, 2, N + 1), [2], dtype)
+    # 32-bit rows into a bfloat16 result: rounded on their way into the matrix instruction
+    both("heads_linear", lambda: (a.float(), w, torch.zeros(T, 2 + H * (N + 1), dtype=torch.bfloat16, device=DEV), 8, K + 8, 2, N + 1),
+         [2], torch.bfloat16)
     one = ops.heads_linear(a[T // 2:T // 2 + 1].contiguous(), w, torch.zeros(1, 2 + H * (N + 1), device=DEV), 8, K + 8, 2, N + 1)
     many = ops.heads_linear(a, w, torch.zeros(T, 2 + H * (N + 1), device=DEV), 8, K + 8, 2, N + 1)
     assert torch.equal(many[T // 2:T // 2 + 1], one), "a row's sums depend on the rows beside it"
