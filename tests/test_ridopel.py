@@ -411,3 +411,60 @@ def test_a_checkpoint_that_does_not_fit_is_reported_whole(folders, tmp_path):
     with pytest.raises(CheckpointError) as e:
         ModelRunner.from_folder(d, EngineOptions(dtype="float32", device="cpu", cache_tokens=64, max_live=1))
     assert "l0.mlp.e1.up" in e.value.missing and "stray" in e.value.unexpected and e.value.wrong_shape[0][0] == "l1.mix.mu.r"
+
+
+# ----------------------------------------------------------------------------------------------------------------
+# the command line and the trace runner as child processes; a long run of decoded tokens
+# ----------------------------------------------------------------------------------------------------------------
+def plain_greedy(folder, prompt, n):
+    seq = list(prompt)
+    for _ in range(n):
+        seq.append(int(plain_logits(folder, seq)[-1].argmax()))
+    return seq[len(prompt):]
+
+
+@pytest.mark.gpu
+def test_command_line_generates_what_the_plain_model_does(folders):
+    import subprocess
+    import sys
+    from conftest import ROOT
+    folder = folders("R", "float32")
+    prompt = seqs_for(CONFIGS["R"][0], [7], seed=410)[0]
+    want = plain_greedy(folder, prompt, 6)
+    out = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "denno"), "generate", folder, "--prompt-ids",
+                          ",".join(map(str, prompt)), "--max-tokens", "6", "--temperature", "0", "--quant", "fp32", "--raw",
+                          "--cache-tokens", "128"], capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0, out.stderr
+    assert [int(t) for t in out.stdout.strip().split(",")] == want
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_run_as_a_child_process(folders, tmp_path, dtype):
+    """bin/trace_run on a mixed trace with four state slots: the files it writes against the plain implementation."""
+    import subprocess
+    from conftest import ROOT
+    cfg = CONFIGS["P"][0] if dtype == "float32" else all_experts(CONFIGS["P"][0])
+    folder = folders("P", dtype, cfg, CONFIGS["P"][1])
+    seqs = seqs_for(cfg, [90, 3, 41, 17, 64, 29, 5], seed=500)
+    steps = U.mixed_trace(seqs, seed=3, max_live=4)
+    out = str(tmp_path / "out")
+    p = subprocess.run([os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype", dtype, "--out", out, "--max-tokens",
+                        str(U.max_live_tokens(steps))], input="\n".join(json.dumps(s) for s in steps) + "\n",
+                       capture_output=True, text=True, timeout=600)
+    assert p.returncode == 0, p.stderr[-2000:]
+    assert [l for l in p.stdout.splitlines() if l.startswith("done ")] == [f"done {s['step']}" for s in steps]
+    got = U.collect_files(out, steps, cfg["vocab"])
+    for i, s in enumerate(seqs):
+        assert_rows(got[f"r{i}"], plain_logits(folder, s), dtype, f"trace_run {dtype} request {i}")
+
+
+def test_two_hundred_decoded_tokens(backend, folders):
+    """A short prompt, then token after token for long: pages fill and new ones are taken, the states run on."""
+    cfg = CONFIGS["P"][0]
+    folder = folders("P", "float32")
+    n = 60 if backend == "cpu" else 230
+    seq = seqs_for(cfg, [n], seed=600)[0]
+    steps = U.tail_decode_trace([seq], n - 4)
+    r = runner_for(folder, "float32", backend, U.max_live_tokens(steps))
+    assert_rows(U.replay(r, steps)["r0"], plain_logits(folder, seq), "float32", "long decoding")
