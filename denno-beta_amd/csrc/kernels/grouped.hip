@@ -1,8 +1,10 @@
 // Products whose weight depends on the row's group: a matrix per head (out[t, h, :] = W_h a[t, h, :]) and a
-// matrix per expert for the rows that a router sent there.  One tile routine serves both: 16 rows x 64 columns a
-// workgroup of 256 threads, K in chunks of 32 through LDS, 32-bit sums in ascending order of k, so a row's result
-// does not depend on which other rows share its tile.  Also the router's choice and the plan that sorts a step's
-// (row, choice) pairs by expert.
+// matrix per expert for the rows that a router sent there; the router's choice and the plan that sorts a step's
+// (row, choice) pairs by expert.  bfloat16 products run on the matrix cores (v_mfma_f32_16x16x32_bf16, operands
+// straight from memory into the lanes that the instruction reads; the experts' matrices packed in that order);
+// 32-bit products, and sizes the matrix-core kernels do not take, run in one tiled vector routine (16 rows x 64
+// columns a workgroup, K in chunks of 32 through LDS).  Every kernel sums an output's k in one ascending order,
+// so a row's result does not depend on which other rows share its tile or on which kernel variant ran.
 #include "common.h"
 
 namespace {
