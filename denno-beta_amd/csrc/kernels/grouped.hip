@@ -352,6 +352,37 @@ __device__ __forceinline__ void mfma_tile(const bf16_t* const a_ptr[2], const bf
   }
 }
 
+// The same with packed W and rows that are gathered (a token's row per pair): a lane asks for the 16 bytes `chunk = l % 4`
+// of row l / 4, so that four neighbouring lanes read one row's 64 bytes (a load then touches 16 cache lines, not 64), and
+// the block goes through a piece of LDS of the wave's own to the lanes that the instruction wants it in (lane l: row
+// l % 16, chunk l / 16).  A wave's LDS accesses run in the order asked, so no barrier stands between the two.
+template <bool DUAL, int CB>
+__device__ __forceinline__ void mfma_tile_staged(bf16x8* stage, const bf16_t* const a_src[2], const bf16_t* const w_ptr[CB],
+                                                 const bf16_t* const w2_ptr[CB], int K, f32x4 acc[2][CB], f32x4 acc2[2][CB]) {
+  const int lane = threadIdx.x & 63;
+  const int put = (lane & 3) * 16 + (lane >> 2);
+#pragma unroll 2
+  for (int k0 = 0; k0 < K; k0 += 32) {
+    bf16x8 af[2], wf[CB], wf2[CB];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) stage[i * 64 + put] = load8(a_src[i] + k0);
+#pragma unroll
+    for (int j = 0; j < CB; ++j) {
+      wf[j] = load8(w_ptr[j] + static_cast<size_t>(k0 / 32) * 512);
+      if (DUAL) wf2[j] = load8(w2_ptr[j] + static_cast<size_t>(k0 / 32) * 512);
+    }
+#pragma unroll
+    for (int i = 0; i < 2; ++i) af[i] = stage[i * 64 + lane];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < CB; ++j) {
+        acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[j], af[i], acc[i][j], 0, 0, 0);
+        if (DUAL) acc2[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf2[j], af[i], acc2[i][j], 0, 0, 0);
+      }
+  }
+}
+
 // Workgroups are handed to the eight XCDs in turn, and each XCD has an L2 of its own: the launch is one line of
 // workgroups, and workgroup L takes the work L' = (L % 8) * (n / 8) + L / 8, so that an XCD gets a run of neighbouring
 // tiles (row tiles fastest: the tiles of one expert and column block, which read the same weights, meet in one L2).
@@ -472,10 +503,12 @@ __global__ __launch_bounds__(256) void expert_up_packed_kernel(const bf16_t* h, 
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int pw = p0 + (wave >> 1) * 32, nw = ty * (32 * CB) + (wave & 1) * (16 * CB);
   if (pw >= p1 || nw >= ff) return;
-  const int kq = (lane >> 4) * 8, lr = lane & 15, ksteps = width / 32;
+  __shared__ bf16x8 stage[4][128];
+  const int lr = lane & 15, ksteps = width / 32;
   const bf16_t *a_ptr[2], *g_ptr[CB], *u_ptr[CB];
 #pragma unroll
-  for (int i = 0; i < 2; ++i) a_ptr[i] = h + static_cast<size_t>(order[min(pw + 16 * i + lr, p1 - 1)] / top) * ldh + kq;
+  for (int i = 0; i < 2; ++i)
+    a_ptr[i] = h + static_cast<size_t>(order[min(pw + 16 * i + (lane >> 2), p1 - 1)] / top) * ldh + (lane & 3) * 8;
 #pragma unroll
   for (int j = 0; j < CB; ++j) {
     const size_t block = (static_cast<size_t>(e) * ff + min(nw + 16 * j, ff - 16)) / 16;
@@ -483,7 +516,7 @@ __global__ __launch_bounds__(256) void expert_up_packed_kernel(const bf16_t* h, 
     u_ptr[j] = wu + block * ksteps * 512 + lane * 8;
   }
   f32x4 g[2][CB] = {}, u[2][CB] = {};
-  mfma_tile<true, true, CB>(a_ptr, g_ptr, u_ptr, width, g, u);
+  mfma_tile_staged<true, CB>(stage[wave], a_ptr, g_ptr, u_ptr, width, g, u);
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
     const int p = pw + 16 * i + lr;
@@ -510,15 +543,16 @@ __global__ __launch_bounds__(256) void expert_down_packed_kernel(const bf16_t* y
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int pw = p0 + (wave >> 1) * 32, nw = ty * (32 * CB) + (wave & 1) * (16 * CB);
   if (pw >= p1 || nw >= width) return;
-  const int kq = (lane >> 4) * 8, lr = lane & 15, ksteps = ff / 32;
+  __shared__ bf16x8 stage[4][128];
+  const int lr = lane & 15, ksteps = ff / 32;
   const bf16_t *a_ptr[2], *w_ptr[CB];
 #pragma unroll
-  for (int i = 0; i < 2; ++i) a_ptr[i] = y + static_cast<size_t>(min(pw + 16 * i + lr, p1 - 1)) * ff + kq;
+  for (int i = 0; i < 2; ++i) a_ptr[i] = y + static_cast<size_t>(min(pw + 16 * i + (lane >> 2), p1 - 1)) * ff + (lane & 3) * 8;
 #pragma unroll
   for (int j = 0; j < CB; ++j)
     w_ptr[j] = wd + (static_cast<size_t>(e) * width + min(nw + 16 * j, width - 16)) / 16 * ksteps * 512 + lane * 8;
   f32x4 acc[2][CB] = {};
-  mfma_tile<false, true, CB>(a_ptr, w_ptr, nullptr, ff, acc, nullptr);
+  mfma_tile_staged<false, CB>(stage[wave], a_ptr, w_ptr, nullptr, ff, acc, nullptr);
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
     const int p = pw + 16 * i + lr;
