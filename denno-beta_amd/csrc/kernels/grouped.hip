@@ -89,10 +89,17 @@ __global__ __launch_bounds__(256) void heads_linear_kernel(const void* A, int a_
 // ---- the router's choice -------------------------------------------------------------------------------------
 // Per row: s = softmax(z) over the experts; the `top` largest of s + correction are chosen (the lower index wins a
 // tie), weighed by their s divided by the sum of the chosen s (+ 1e-20).  A thread a row.
-__global__ __launch_bounds__(64) void route_kernel(const float* z, const float* correction, int T, int E, int top, int* ids, float* wts) {
+// (sigmoid: the scores are s = 1 / (1 + e^-z), each expert's own; renorm 0: the weights are the chosen scores as they are.
+// A row of z may be wider than the experts: rows are ldz numbers apart.)
+__device__ __forceinline__ float route_score(bool sigmoid, float z, float m, float sum) {
+  return sigmoid ? 1.0f / (1.0f + expf(-z)) : expf(z - m) / sum;
+}
+
+__global__ __launch_bounds__(64) void route_kernel(const float* z, size_t ldz, const float* correction, int T, int E, int top,
+                                                   int sigmoid, int renorm, int* ids, float* wts) {
   const int t = blockIdx.x * 64 + threadIdx.x;
   if (t >= T) return;
-  const float* row = z + static_cast<size_t>(t) * E;
+  const float* row = z + static_cast<size_t>(t) * ldz;
   float m = row[0];
   for (int e = 1; e < E; ++e) m = fmaxf(m, row[e]);
   float sum = 0.f;
@@ -105,7 +112,7 @@ __global__ __launch_bounds__(64) void route_kernel(const float* z, const float* 
       bool taken = false;
       for (int q = 0; q < c; ++q) taken |= ids[t * top + q] == e;
       if (taken) continue;
-      const float sc = expf(row[e] - m) / sum;
+      const float sc = route_score(sigmoid, row[e], m, sum);
       const float v = sc + (correction ? correction[e] : 0.f);
       if (best < 0 || v > best_v) best = e, best_v = v, best_s = sc;
     }
@@ -113,15 +120,17 @@ __global__ __launch_bounds__(64) void route_kernel(const float* z, const float* 
     wts[t * top + c] = best_s;
     chosen_sum += best_s;
   }
+  if (!renorm) return;
   const float inv = 1.0f / (chosen_sum + 1e-20f);
   for (int c = 0; c < top; ++c) wts[t * top + c] *= inv;
 }
 
 // The same choice with a wave a row (up to 8,192 experts, `top` up to 64): lane l has the experts l, l + 64, ...; the
 // largest score is found over the lanes, the lowest index among equals wins, and lane c keeps the c-th choice.
-__global__ __launch_bounds__(64) void route_wave_kernel(const float* z, const float* correction, int E, int top, int* ids, float* wts) {
+__global__ __launch_bounds__(64) void route_wave_kernel(const float* z, size_t ldz, const float* correction, int E, int top, int sigmoid,
+                                                        int renorm, int* ids, float* wts) {
   const int t = blockIdx.x, lane = threadIdx.x;
-  const float* row = z + static_cast<size_t>(t) * E;
+  const float* row = z + static_cast<size_t>(t) * ldz;
   const float none = -__builtin_huge_valf();
   float m = none;
   for (int e = lane; e < E; e += 64) m = fmaxf(m, row[e]);
@@ -137,7 +146,7 @@ __global__ __launch_bounds__(64) void route_wave_kernel(const float* z, const fl
     int best = 0x7fffffff;
     for (int e = lane, k = 0; e < E; e += 64, ++k) {
       if ((taken[k >> 5] >> (k & 31)) & 1u) continue;
-      const float sc = expf(row[e] - m) / sum;
+      const float sc = route_score(sigmoid, row[e], m, sum);
       const float v = sc + (correction ? correction[e] : 0.f);
       if (v > best_v) best_v = v, best = e, best_s = sc;
     }
@@ -152,7 +161,7 @@ __global__ __launch_bounds__(64) void route_wave_kernel(const float* z, const fl
   const float chosen = wave_sum(lane < top ? my_w : 0.f);
   if (lane < top) {
     ids[t * top + lane] = my_id;
-    wts[t * top + lane] = my_w / (chosen + 1e-20f);
+    wts[t * top + lane] = renorm ? my_w / (chosen + 1e-20f) : my_w;
   }
 }
 
@@ -249,10 +258,28 @@ __device__ __forceinline__ bool expert_tile(const int* offsets, int E, int id, i
   return false;
 }
 
-// ---- an expert's first half: y[p, :] = g * sigmoid(alpha g) * (u + 1), g = min(W_gate h, limit), u = clamp(W_up h, +-limit) --
+// ---- an expert's first half: y[p, :] = act(W_gate h, W_up h) ---------------------------------------------------
+// kind 0: g * sigmoid(alpha g) * (u + 1) with g = min(W_gate h, limit), u = clamp(W_up h, +-limit)
+// kind 1: silu(s g) * (s u), s the pair's own factor (in_scale[pair]; none: 1): the expert reads s h, and both products
+//         are linear in what they read
+struct ExpertAct {
+  float limit, alpha;
+  int kind;
+  const float* in_scale;
+};
+
+__device__ __forceinline__ float expert_act(const ExpertAct& a, float g, float u, float s) {
+  if (a.kind == 1) {
+    const float gs = g * s;
+    return gs / (1.0f + expf(-gs)) * (u * s);
+  }
+  const float gv = fminf(g, a.limit), uv = fminf(fmaxf(u, -a.limit), a.limit);
+  return gv / (1.0f + expf(-a.alpha * gv)) * (uv + 1.0f);
+}
+
 __global__ __launch_bounds__(256) void expert_up_kernel(const void* h, int h_dt, size_t ldh, const int* order, const int* offsets,
                                                         int E, int top, const void* wg, const void* wu, int w_dt, int ff, int width,
-                                                        float limit, float alpha, void* y, int y_dt) {
+                                                        ExpertAct act, void* y, int y_dt) {
   __shared__ Tile lds, lds2;
   int e, p0, p1;
   if (!expert_tile(offsets, E, blockIdx.x, e, p0, p1)) return;
@@ -267,12 +294,12 @@ __global__ __launch_bounds__(256) void expert_up_kernel(const void* h, int h_dt,
   tile_product<true>(lds, &lds2, h, h_dt, a_row, wg, wu, w_dt, static_cast<size_t>(e) * ff * width, ff, width, n0, g, u);
   const int p = p0 + (tid >> 4);
   if (p >= p1) return;
+  const float sc = act.in_scale ? act.in_scale[order[p]] : 1.0f;
 #pragma unroll
   for (int c = 0; c < 4; ++c) {
     const int n = n0 + (tid & 15) * 4 + c;
     if (n >= ff) continue;
-    const float gv = fminf(g[c], limit), uv = fminf(fmaxf(u[c], -limit), limit);
-    store_as(y, static_cast<size_t>(p) * ff + n, y_dt, gv / (1.0f + expf(-alpha * gv)) * (uv + 1.0f));
+    store_as(y, static_cast<size_t>(p) * ff + n, y_dt, expert_act(act, g[c], u[c], sc));
   }
 }
 
@@ -301,12 +328,12 @@ __global__ __launch_bounds__(256) void expert_down_kernel(const void* y, int y_d
   }
 }
 
-// x[t, :] += sum_c wts[t, c] * out[t * top + c, :], the choices in their order
+// x[t, :] += sum_c wts[t, c] * out[t * top + c, :], the choices in their order (wts none: every weight is 1)
 __global__ __launch_bounds__(256) void combine_kernel(const float* out, const float* wts, int top, int width, float* x, size_t ldx) {
   const int t = blockIdx.x;
   for (int c = threadIdx.x; c < width; c += 256) {
     float acc = 0.f;
-    for (int q = 0; q < top; ++q) acc = fmaf(wts[t * top + q], out[(static_cast<size_t>(t) * top + q) * width + c], acc);
+    for (int q = 0; q < top; ++q) acc = fmaf(wts ? wts[t * top + q] : 1.0f, out[(static_cast<size_t>(t) * top + q) * width + c], acc);
     x[t * ldx + c] += acc;
   }
 }
@@ -420,7 +447,7 @@ __device__ __forceinline__ bool expert_tile64(const int* offsets, int E, int id,
 
 __global__ __launch_bounds__(256) void expert_up_mfma_kernel(const bf16_t* h, size_t ldh, const int* order, const int* offsets, int E,
                                                              int top, const bf16_t* wg, const bf16_t* wu, int ff, int width,
-                                                             float limit, float alpha, bf16_t* y, int tiles_x) {
+                                                             ExpertAct act, bf16_t* y, int tiles_x) {
   int e, p0, p1, tx, ty;
   xcd_tile(tiles_x, (ff + 63) / 64, tx, ty);
   if (tx < 0 || !expert_tile64(offsets, E, tx, e, p0, p1)) return;
@@ -443,14 +470,14 @@ __global__ __launch_bounds__(256) void expert_up_mfma_kernel(const bf16_t* h, si
   for (int i = 0; i < 2; ++i) {
     const int p = pw + 16 * i + lr;
     if (p >= p1) continue;
+    const float sc = act.in_scale ? act.in_scale[order[p]] : 1.0f;
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
       const int n = nw + 16 * j + (lane >> 4) * 4;
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         if (n + r >= ff) continue;
-        const float gv = fminf(g[i][j][r], limit), uv = fminf(fmaxf(u[i][j][r], -limit), limit);
-        y[static_cast<size_t>(p) * ff + n + r] = from_float<bf16_t>(gv / (1.0f + expf(-alpha * gv)) * (uv + 1.0f));
+        y[static_cast<size_t>(p) * ff + n + r] = from_float<bf16_t>(expert_act(act, g[i][j][r], u[i][j][r], sc));
       }
     }
   }
@@ -496,7 +523,7 @@ __global__ __launch_bounds__(256) void expert_down_mfma_kernel(const bf16_t* y, 
 template <int CB>
 __global__ __launch_bounds__(256) void expert_up_packed_kernel(const bf16_t* h, size_t ldh, const int* order, const int* offsets, int E,
                                                                int top, const bf16_t* wg, const bf16_t* wu, int ff, int width,
-                                                               float limit, float alpha, bf16_t* y, int tiles_x) {
+                                                               ExpertAct act, bf16_t* y, int tiles_x) {
   int e, p0, p1, tx, ty;
   xcd_tile(tiles_x, (ff + 32 * CB - 1) / (32 * CB), tx, ty);
   if (tx < 0 || !expert_tile64(offsets, E, tx, e, p0, p1)) return;
@@ -521,15 +548,14 @@ __global__ __launch_bounds__(256) void expert_up_packed_kernel(const bf16_t* h, 
   for (int i = 0; i < 2; ++i) {
     const int p = pw + 16 * i + lr;
     if (p >= p1) continue;
+    const float sc = act.in_scale ? act.in_scale[order[p]] : 1.0f;
 #pragma unroll
     for (int j = 0; j < CB; ++j) {
       const int n = nw + 16 * j + (lane >> 4) * 4;
       if (n >= ff) continue;      // (ff is a multiple of 16: a block is whole or absent)
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const float gv = fminf(g[i][j][r], limit), uv = fminf(fmaxf(u[i][j][r], -limit), limit);
-        y[static_cast<size_t>(p) * ff + n + r] = from_float<bf16_t>(gv / (1.0f + expf(-alpha * gv)) * (uv + 1.0f));
-      }
+      for (int r = 0; r < 4; ++r)
+        y[static_cast<size_t>(p) * ff + n + r] = from_float<bf16_t>(expert_act(act, g[i][j][r], u[i][j][r], sc));
     }
   }
 }
@@ -652,14 +678,17 @@ int dn_heads_linear(const void* a, int a_dt, long long lda, int a_off, int a_str
   return dn_launch_status();
 }
 
-int dn_moe_route(const float* z, const float* correction, int T, int E, int top, int* ids, float* wts, hipStream_t stream) {
-  if (E < 1 || top < 1 || top > E) return DN_ERR_SHAPE;
+int dn_moe_route(const float* z, long long ldz, const float* correction, int T, int E, int top, int sigmoid, int renorm, int* ids,
+                 float* wts, hipStream_t stream) {
+  if (E < 1 || top < 1 || top > E || ldz < E) return DN_ERR_SHAPE;
   if (T == 0) return 0;
   if (E <= 8192 && top <= 64) {
-    hipLaunchKernelGGL(route_wave_kernel, dim3(T), dim3(64), 0, stream, z, correction, E, top, ids, wts);
+    hipLaunchKernelGGL(route_wave_kernel, dim3(T), dim3(64), 0, stream, z, static_cast<size_t>(ldz), correction, E, top, sigmoid, renorm,
+                       ids, wts);
     return dn_launch_status();
   }
-  hipLaunchKernelGGL(route_kernel, dim3((T + 63) / 64), dim3(64), 0, stream, z, correction, T, E, top, ids, wts);
+  hipLaunchKernelGGL(route_kernel, dim3((T + 63) / 64), dim3(64), 0, stream, z, static_cast<size_t>(ldz), correction, T, E, top, sigmoid,
+                     renorm, ids, wts);
   return dn_launch_status();
 }
 
@@ -673,10 +702,12 @@ int dn_moe_plan(const int* ids, int n, int E, int* offsets, int* order, hipStrea
 }
 
 int dn_moe_up(const void* h, int h_dt, long long ldh, const int* order, const int* offsets, int E, int top, int n, const void* wg,
-              const void* wu, int w_dt, int ff, int width, float limit, float alpha, void* y, int y_dt, int packed,
-              hipStream_t stream) {
+              const void* wu, int w_dt, int ff, int width, float limit, float alpha, int kind, const float* in_scale, void* y,
+              int y_dt, int packed, hipStream_t stream) {
   if (!float_kind(h_dt) || !float_kind(w_dt) || !float_kind(y_dt)) return DN_ERR_DTYPE;
+  if (kind < 0 || kind > 1) return DN_ERR_SHAPE;
   if (n == 0) return 0;
+  const ExpertAct act{limit, alpha, kind, in_scale};
   if (packed) {
     if (h_dt != DN_BF16 || w_dt != DN_BF16 || y_dt != DN_BF16) return DN_ERR_DTYPE;
     if (width % 32 != 0 || ff % 16 != 0 || ldh % 8 != 0 || !aligned16(h) || !aligned16(wg) || !aligned16(wu)) return DN_ERR_SHAPE;
@@ -685,12 +716,12 @@ int dn_moe_up(const void* h, int h_dt, long long ldh, const int* order, const in
       const int tiles = tiles_x * ((ff + 31) / 32);
       hipLaunchKernelGGL(expert_up_packed_kernel<1>, dim3((tiles + 7) / 8 * 8), dim3(256), 0, stream, static_cast<const bf16_t*>(h),
                          static_cast<size_t>(ldh), order, offsets, E, top, static_cast<const bf16_t*>(wg),
-                         static_cast<const bf16_t*>(wu), ff, width, limit, alpha, static_cast<bf16_t*>(y), tiles_x);
+                         static_cast<const bf16_t*>(wu), ff, width, act, static_cast<bf16_t*>(y), tiles_x);
     } else {
       const int tiles = tiles_x * ((ff + 127) / 128);
       hipLaunchKernelGGL(expert_up_packed_kernel<4>, dim3((tiles + 7) / 8 * 8), dim3(256), 0, stream, static_cast<const bf16_t*>(h),
                          static_cast<size_t>(ldh), order, offsets, E, top, static_cast<const bf16_t*>(wg),
-                         static_cast<const bf16_t*>(wu), ff, width, limit, alpha, static_cast<bf16_t*>(y), tiles_x);
+                         static_cast<const bf16_t*>(wu), ff, width, act, static_cast<bf16_t*>(y), tiles_x);
     }
     return dn_launch_status();
   }
@@ -699,11 +730,11 @@ int dn_moe_up(const void* h, int h_dt, long long ldh, const int* order, const in
     const int tiles_x = (n + MT - 1) / MT + E, tiles = tiles_x * ((ff + 63) / 64);
     hipLaunchKernelGGL(expert_up_mfma_kernel, dim3((tiles + 7) / 8 * 8), dim3(256), 0, stream,
                        static_cast<const bf16_t*>(h), static_cast<size_t>(ldh), order, offsets, E, top, static_cast<const bf16_t*>(wg),
-                       static_cast<const bf16_t*>(wu), ff, width, limit, alpha, static_cast<bf16_t*>(y), tiles_x);
+                       static_cast<const bf16_t*>(wu), ff, width, act, static_cast<bf16_t*>(y), tiles_x);
     return dn_launch_status();
   }
   hipLaunchKernelGGL(expert_up_kernel, dim3((n + TM - 1) / TM + E, (ff + TN - 1) / TN), dim3(256), 0, stream, h, h_dt,
-                     static_cast<size_t>(ldh), order, offsets, E, top, wg, wu, w_dt, ff, width, limit, alpha, y, y_dt);
+                     static_cast<size_t>(ldh), order, offsets, E, top, wg, wu, w_dt, ff, width, act, y, y_dt);
   return dn_launch_status();
 }
 

@@ -1,12 +1,15 @@
 // Kernels for layers that carry something from token to token besides keys and values: norms without a
 // mean, short causal convolutions over time, the previous token's row, turned pairs of dimensions, and
-// matrix states that decay (one scan for every recurrence of the form S <- diag(w) S + a v^T).
+// matrix states that decay (one scan for every recurrence of the form S <- diag(w) S + a v^T, and for the delta rule,
+// which writes what the state does not yet answer to a key), norms that add into the stream, averages over depth.
 // Everything here is 32-bit arithmetic; only what is read or stored may be bfloat16.  A request's rows
 // are rows row_start[s] .. row_start[s + 1] - 1 of the step, its state lies at slots[s]; a request whose
 // slot is negative is padding and is skipped.
 #include "common.h"
 
 namespace {
+
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
 
 __device__ __forceinline__ float load_as(const void* p, size_t i, int dt) {
   return dt == DN_F32 ? static_cast<const float*>(p)[i] : to_float(static_cast<const bf16_t*>(p)[i]);
@@ -57,6 +60,50 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const void* x, int x_dt, s
   }
 }
 
+// x[t, :] += mult * (y[t, :] / sqrt(mean(y^2) + eps) * weight) * scale: the norm of a sublayer's result, added into the
+// stream (scale: a vector, or none).  One workgroup a row, the sums as in rmsnorm_kernel.
+__global__ __launch_bounds__(256) void rmsnorm_add_kernel(const void* y, int y_dt, size_t ldy, const float* weight, const float* scale,
+                                                          float mult, float* x, size_t ldx, int width, float eps) {
+  __shared__ float sh[4];
+  const size_t src = static_cast<size_t>(blockIdx.x) * ldy, dst = static_cast<size_t>(blockIdx.x) * ldx;
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < width; c += 256) {
+    const float v = load_as(y, src + c, y_dt);
+    ss = fmaf(v, v, ss);
+  }
+  ss = block_sum_256(ss, sh);
+  const float inv = 1.0f / sqrtf(ss / static_cast<float>(width) + eps);
+  for (int c = threadIdx.x; c < width; c += 256) {
+    float v = load_as(y, src + c, y_dt) * inv;
+    if (weight) v *= weight[c];
+    if (scale) v *= scale[c];
+    x[dst + c] = fmaf(mult, v, x[dst + c]);
+  }
+}
+
+// out[i] = sum_j w[j] * hist[j][i], j ascending from 0 to n - 1, one fused multiply-add a step: an average over the
+// streams that the layers so far have left ([n][rows * width], `plane` numbers apart).  out may be a later plane.
+__global__ __launch_bounds__(256) void depth_mix_kernel(const float* hist, size_t plane, int n, const float* w, float* out, size_t total,
+                                                        int vec) {
+  const size_t i = (static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x) * 4;
+  if (i >= total) return;
+  if (vec && i + 4 <= total) {
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    for (int j = 0; j < n; ++j) {
+      const f32x4 v = *reinterpret_cast<const f32x4*>(hist + j * plane + i);
+      const float wj = w[j];
+      acc[0] = fmaf(wj, v[0], acc[0]), acc[1] = fmaf(wj, v[1], acc[1]), acc[2] = fmaf(wj, v[2], acc[2]), acc[3] = fmaf(wj, v[3], acc[3]);
+    }
+    *reinterpret_cast<f32x4*>(out + i) = acc;
+  } else {
+    for (size_t e = i; e < total && e < i + 4; ++e) {
+      float acc = 0.f;
+      for (int j = 0; j < n; ++j) acc = fmaf(w[j], hist[j * plane + e], acc);
+      out[e] = acc;
+    }
+  }
+}
+
 // out[t, :] = [a[t, :wa] | b[t, :wb]]
 __global__ __launch_bounds__(256) void concat_kernel(const float* a, size_t lda, int wa, const float* b, size_t ldb, int wb,
                                                      void* out, int out_dt) {
@@ -67,33 +114,36 @@ __global__ __launch_bounds__(256) void concat_kernel(const float* a, size_t lda,
 }
 
 // ---- short causal convolution over time ----------------------------------------------------------------------
-// out[t, c] = h[t, c] + sum_j w[c, j] * h[t - taps + 1 + j, c]; rows before the step's first row of a request come
-// from its history [slot][taps - 1][width] (oldest first; zero for a new request).
-__global__ __launch_bounds__(256) void conv_rows_kernel(const float* h, const float* w, const float* hist, const int* row_start,
-                                                        const int* slots, int S, int width, int taps, void* out, int out_dt, size_t hist_stride) {
+// out[t, c] = act((identity ? h[t, c] : 0) + sum_j w[c, j] * h[t - taps + 1 + j, c]); rows before the step's first row of a
+// request come from its history [slot][taps - 1][width] (oldest first; zero for a new request).  h and out are rows
+// ldh and ldo numbers apart (the channels may be the first columns of wider rows); act: none or silu.
+__global__ __launch_bounds__(256) void conv_rows_kernel(const float* h, size_t ldh, const float* w, const float* hist, const int* row_start,
+                                                        const int* slots, int S, int width, int taps, int identity, int silu, void* out,
+                                                        int out_dt, size_t ldo, size_t hist_stride) {
   const int t = blockIdx.x;
   const int s = request_of(row_start, S, t);
   const int slot = slots[s];
   if (slot < 0 || t >= row_start[S]) {      // a padding row: zeros, so that what follows works on numbers
-    for (int c = threadIdx.x; c < width; c += 256) store_as(out, static_cast<size_t>(t) * width + c, out_dt, 0.f);
+    for (int c = threadIdx.x; c < width; c += 256) store_as(out, static_cast<size_t>(t) * ldo + c, out_dt, 0.f);
     return;
   }
   const int i = t - row_start[s];
   const float* past = hist + static_cast<size_t>(slot) * hist_stride;
   for (int c = threadIdx.x; c < width; c += 256) {
-    float acc = h[static_cast<size_t>(t) * width + c];
+    float acc = identity ? h[static_cast<size_t>(t) * ldh + c] : 0.f;
     for (int j = 0; j < taps; ++j) {
       const int src = i - taps + 1 + j;
-      const float v = src >= 0 ? h[static_cast<size_t>(row_start[s] + src) * width + c] : past[static_cast<size_t>(i + j) * width + c];
+      const float v = src >= 0 ? h[static_cast<size_t>(row_start[s] + src) * ldh + c] : past[static_cast<size_t>(i + j) * width + c];
       acc = fmaf(w[c * taps + j], v, acc);
     }
-    store_as(out, static_cast<size_t>(t) * width + c, out_dt, acc);
+    if (silu) acc = acc / (1.0f + expf(-acc));
+    store_as(out, static_cast<size_t>(t) * ldo + c, out_dt, acc);
   }
 }
 
 // The last `keep` rows of (history ++ this step's rows) become the history.  A thread owns a channel of a request and
 // goes through the places in ascending order: place m reads the old place m + n, which it has not written yet.
-__global__ __launch_bounds__(256) void history_update_kernel(const void* h, int h_dt, float* hist, const int* row_start,
+__global__ __launch_bounds__(256) void history_update_kernel(const void* h, int h_dt, size_t ldh, float* hist, const int* row_start,
                                                              const int* slots, int width, int keep, size_t hist_stride) {
   const int s = blockIdx.x;
   const int slot = slots[s];
@@ -104,7 +154,7 @@ __global__ __launch_bounds__(256) void history_update_kernel(const void* h, int 
     for (int m = 0; m < keep; ++m) {
       const int src = n - keep + m;
       past[static_cast<size_t>(m) * width + c] =
-          src >= 0 ? load_as(h, static_cast<size_t>(row0 + src) * width + c, h_dt) : past[static_cast<size_t>(m + n) * width + c];
+          src >= 0 ? load_as(h, static_cast<size_t>(row0 + src) * ldh + c, h_dt) : past[static_cast<size_t>(m + n) * width + c];
     }
 }
 
@@ -159,12 +209,16 @@ __global__ __launch_bounds__(256) void rotary_kernel(const void* src, int src_dt
 }
 
 // ---- activations of projections that feed a recurrence or a gate --------------------------------------------
-enum { ACT_SILU = 0, ACT_SIGMOID = 1, ACT_TANH = 2, ACT_EXP_NEG_EXP = 3, ACT_BOUNDED_SIGMOID = 4 };
+enum { ACT_SILU = 0, ACT_SIGMOID = 1, ACT_TANH = 2, ACT_EXP_NEG_EXP = 3, ACT_BOUNDED_SIGMOID = 4, ACT_EXP_NEG_SOFTPLUS = 5, ACT_XIELU = 6 };
 
 __device__ __forceinline__ float sigmoid_f(float z) { return 1.0f / (1.0f + expf(-z)); }
 
+// log(1 + e^z), without overflow
+__device__ __forceinline__ float softplus_f(float z) { return fmaxf(z, 0.f) + log1pf(expf(-fabsf(z))); }
+
 __device__ __forceinline__ float activation(int kind, float z, float lower) {
   switch (kind) {
+    case ACT_EXP_NEG_SOFTPLUS: return expf(-lower * softplus_f(z));      // (lower: the rate of the column)
     case ACT_SILU: return z * sigmoid_f(z);
     case ACT_SIGMOID: return sigmoid_f(z);
     case ACT_TANH: return tanhf(z);
@@ -173,14 +227,34 @@ __device__ __forceinline__ float activation(int kind, float z, float lower) {
   }
 }
 
-// out[t, c] = act(x[t, c] + bias[c]) (lower[c]: the least value of a bounded sigmoid)
+// out[t, c] = act(x[t, c] + bias[c]) (lower[c]: the least value of a bounded sigmoid, or the rate of exp(-rate softplus(z)));
+// "xielu" has two numbers for all columns in `lower`, (a, b): z > 0: a z^2 + z / 2; else b (e^z - 1 - z) + z / 2
 __global__ __launch_bounds__(256) void activate_kernel(const float* x, size_t ldx, const float* bias, const float* lower, int kind,
                                                        void* out, int out_dt, size_t ldo, int n) {
   const int t = blockIdx.x;
+  if (kind == ACT_XIELU) {
+    const float a = lower[0], b = lower[1];
+    for (int c = threadIdx.x; c < n; c += 256) {
+      const float z = x[t * ldx + c] + (bias ? bias[c] : 0.f);
+      store_as(out, t * ldo + c, out_dt, z > 0.f ? fmaf(a * z, z, 0.5f * z) : fmaf(b, expm1f(z) - z, 0.5f * z));
+    }
+    return;
+  }
   for (int c = threadIdx.x; c < n; c += 256) {
     const float z = x[t * ldx + c] + (bias ? bias[c] : 0.f);
     store_as(out, t * ldo + c, out_dt, activation(kind, z, lower ? lower[c] : 0.f));
   }
+}
+
+// out[t, h, :] = x[t, h, :] / sqrt(sum(x[t, h, :]^2) + eps) * scale: every head's vector made a unit vector; a wave a head
+__global__ __launch_bounds__(64) void unit_heads_kernel(const float* x, size_t ldx, float* out, size_t ldo, int dim, float eps, float scale) {
+  const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const float* src = x + t * ldx + static_cast<size_t>(h) * dim;
+  float ss = 0.f;
+  for (int j = lane; j < dim; j += 64) ss = fmaf(src[j], src[j], ss);
+  ss = wave_sum(ss);
+  const float inv = scale / sqrtf(ss + eps);
+  for (int j = lane; j < dim; j += 64) out[t * ldo + static_cast<size_t>(h) * dim + j] = src[j] * inv;
 }
 
 // out[t, c] = x[t, c] * act(g[t, c])
@@ -196,7 +270,10 @@ __global__ __launch_bounds__(256) void gated_kernel(const void* x, int x_dt, siz
 // walks the request's rows of this step in order:
 //   a_i = key_from_decay ? 1 - w_i : k_i
 //   read_after:   S_i <- w_i S_i + a_i v_j ;  o_j = sum_i r_i S_i
+//   delta:        S_i <- w_i S_i ;  e_j = beta (v_j - sum_i a_i S_i) ;  S_i <- S_i + a_i e_j ;  o_j = sum_i r_i S_i
 //   else:         o_j = sum_i r_i (S_i + u_i a_i v_j) ;  S_i <- w_i S_i + a_i v_j
+// w is a number per row, head and key channel, or (w_head) one per head for all rows and channels.  r and k may have
+// fewer heads than v: head h reads r and k of head h / (H / G).
 // A column's key channels are shared out among KG lanes that lie side by side (4 lanes for heads of up to 32 key
 // channels, 16 beyond), so a wave has 64 / KG columns and a column's parts are joined inside a row of 16 lanes,
 // without LDS; a part's sum over i runs in ascending order, one fused multiply-add a step, and the parts are joined
@@ -204,11 +281,12 @@ __global__ __launch_bounds__(256) void gated_kernel(const void* x, int x_dt, siz
 // A row's r, k and w reach the lanes through LDS, some rows at a time (16, or 2 in a step of single rows); the next are asked for before the
 // current ones are worked on.  Places beyond a request's last row hold r = 0, a = 0, w = 1, which change nothing, so the
 // rows of a fetch are worked on without a branch between them.
-typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
+enum { SCAN_BEFORE = 0, SCAN_AFTER = 1, SCAN_DELTA = 2 };
 
 struct ScanArgs {
-  const float *r, *k, *v, *w, *u;
-  size_t ldr, ldk, ldv, ldw;
+  const float *r, *k, *v, *w, *u, *beta, *w_head;
+  size_t ldr, ldk, ldv, ldw, ldb;
+  int G;
   float* state;
   size_t slot_stride;
   const int *row_start, *slots;
@@ -217,8 +295,9 @@ struct ScanArgs {
   size_t ldo;
 };
 
-template <int DK, int KG, bool AFTER, bool VEC, int TB>
+template <int DK, int KG, int MODE, bool VEC, int TB>
 __global__ __launch_bounds__(64) void scan_kernel(ScanArgs a) {
+  constexpr bool AFTER = MODE == SCAN_AFTER, DELTA = MODE == SCAN_DELTA;
   constexpr int KQ = DK / KG;
   constexpr int CW = 64 / KG;      // value columns of a wave
   constexpr int NL = DK >= 64 ? DK / 64 : 1;
@@ -228,7 +307,10 @@ __global__ __launch_bounds__(64) void scan_kernel(ScanArgs a) {
   __shared__ __attribute__((aligned(16))) float sh[TB][3 * DK];
   __shared__ __attribute__((aligned(16))) float shv[TB][CW];
   __shared__ __attribute__((aligned(16))) float shu[DK];
+  __shared__ float shb[TB];
   const int s = blockIdx.z, h = blockIdx.y, lane = threadIdx.x;
+  const int hq = h / (a.H / a.G);                     // the head of r and k that this head reads
+  const float wh = a.w_head ? a.w_head[h] : 1.0f;     // one decay for the head, where w is none
   const int kg = lane % KG, j0 = blockIdx.x * CW, j = j0 + lane / KG;
   const int slot = a.slots[s];
   if (slot < 0) return;
@@ -245,7 +327,7 @@ __global__ __launch_bounds__(64) void scan_kernel(ScanArgs a) {
   // what a fetch brings: (not VEC) a lane's own numbers row by row; (VEC: every size a multiple of 4 and every row at a
   // multiple of 16 bytes) 16 bytes a lane and load, eight rows of r, k or w in DK / 32 loads: a row then costs a wave
   // 7 / 8 of a vector load where it cost four, and those loads, not the arithmetic, were what a row waited for
-  float nr[VEC ? 1 : TB][NL], nk[VEC ? 1 : TB][NL], nw[VEC ? 1 : TB][NL], nv[VEC ? 1 : TB];
+  float nr[VEC ? 1 : TB][NL], nk[VEC ? 1 : TB][NL], nw[VEC ? 1 : TB][NL], nv[VEC ? 1 : TB], nb[VEC ? 1 : TB];
   f32x4 r4[VEC ? NV : 1], k4[VEC ? NV : 1], w4[VEC ? NV : 1], v4;
   auto fetch = [&](int t0) {
     if constexpr (VEC) {
@@ -254,10 +336,11 @@ __global__ __launch_bounds__(64) void scan_kernel(ScanArgs a) {
       for (int it = 0; it < NV; ++it) {
         const int idx = it * 64 + lane, bq = idx / (DK / 4), i = (idx % (DK / 4)) * 4, t = t0 + bq;
         const bool ok = idx < N4 && t < row1 && i < dk;
-        r4[it] = ok ? *reinterpret_cast<const f32x4*>(a.r + t * a.ldr + h * dk + i) : zero;
-        k4[it] = (ok && !a.key_from_decay) ? *reinterpret_cast<const f32x4*>(a.k + t * a.ldk + h * dk + i) : zero;
-        w4[it] = ok ? *reinterpret_cast<const f32x4*>(a.w + t * a.ldw + h * dk + i) : one;
+        r4[it] = ok ? *reinterpret_cast<const f32x4*>(a.r + t * a.ldr + hq * dk + i) : zero;
+        k4[it] = (ok && !a.key_from_decay) ? *reinterpret_cast<const f32x4*>(a.k + t * a.ldk + hq * dk + i) : zero;
+        w4[it] = !ok ? one : a.w_head ? one * wh : *reinterpret_cast<const f32x4*>(a.w + t * a.ldw + h * dk + i);
       }
+      if constexpr (DELTA) nb[0] = (lane < TB && t0 + lane < row1) ? a.beta[(t0 + lane) * a.ldb + h] : 0.f;
       const int bq = lane / (CW / 4), col = j0 + (lane % (CW / 4)) * 4, t = t0 + bq;
       v4 = (lane < TB * CW / 4 && t < row1 && col < dv) ? *reinterpret_cast<const f32x4*>(a.v + t * a.ldv + h * dv + col) : zero;
     } else {
@@ -269,18 +352,22 @@ __global__ __launch_bounds__(64) void scan_kernel(ScanArgs a) {
         for (int q = 0; q < NL; ++q) {
           const int i = lane + 64 * q;
           const bool ok = row && i < dk;
-          nr[bq][q] = ok ? a.r[t * a.ldr + h * dk + i] : 0.f;
-          nk[bq][q] = (ok && !a.key_from_decay) ? a.k[t * a.ldk + h * dk + i] : 0.f;
-          nw[bq][q] = ok ? a.w[t * a.ldw + h * dk + i] : 1.f;
+          nr[bq][q] = ok ? a.r[t * a.ldr + hq * dk + i] : 0.f;
+          nk[bq][q] = (ok && !a.key_from_decay) ? a.k[t * a.ldk + hq * dk + i] : 0.f;
+          nw[bq][q] = !ok ? 1.f : a.w_head ? wh : a.w[t * a.ldw + h * dk + i];
         }
+        if constexpr (DELTA) nb[bq] = row ? a.beta[t * a.ldb + h] : 0.f;
         nv[bq] = (row && live) ? a.v[t * a.ldv + h * dv + j] : 0.f;
       }
     }
   };
   fetch(row0);
   for (int t0 = row0; t0 < row1; t0 += TB) {
-    float vj[TB];
+    float vj[TB], bj[TB];
     if constexpr (VEC) {
+      if constexpr (DELTA) {
+        if (lane < TB) shb[lane] = nb[0];
+      }
 #pragma unroll
       for (int it = 0; it < NV; ++it) {
         const int idx = it * 64 + lane, bq = idx / (DK / 4), i = (idx % (DK / 4)) * 4;
@@ -305,12 +392,16 @@ __global__ __launch_bounds__(64) void scan_kernel(ScanArgs a) {
           }
         }
         vj[bq] = nv[bq];
+        if constexpr (DELTA) bj[bq] = nb[bq];
       }
     }
     __syncthreads();
     if constexpr (VEC) {
 #pragma unroll
-      for (int bq = 0; bq < TB; ++bq) vj[bq] = shv[bq][lane / KG];
+      for (int bq = 0; bq < TB; ++bq) {
+        vj[bq] = shv[bq][lane / KG];
+        if constexpr (DELTA) bj[bq] = shb[bq];
+      }
     }
     if (t0 + TB < row1) fetch(t0 + TB);
     // (no branch inside the eight rows: their reads, sums and joins can then overlap)
@@ -322,6 +413,24 @@ __global__ __launch_bounds__(64) void scan_kernel(ScanArgs a) {
       const float* mw = mk + DK;
       const float* mu = shu + kg * KQ;
       float o = 0.f;
+      if constexpr (DELTA) {
+        // the state fades; what it answers to the key is taken off the value; the rest, times beta, is written
+        float ans = 0.f;
+#pragma unroll
+        for (int q = 0; q < KQ; ++q) {
+          S[q] *= mw[q];
+          ans = fmaf(mk[q], S[q], ans);
+        }
+        ans = group_reduce<KG>(ans, SumOp());
+        const float e = bj[bq] * (vj[bq] - ans);
+#pragma unroll
+        for (int q = 0; q < KQ; ++q) {
+          S[q] = fmaf(mk[q], e, S[q]);
+          o = fmaf(mr[q], S[q], o);
+        }
+        ob[bq] = group_reduce<KG>(o, SumOp());
+        continue;
+      }
 #pragma unroll
       for (int q = 0; q < KQ; ++q) {
         const float kv = mk[q] * vj[bq];
@@ -383,6 +492,35 @@ int dn_rmsnorm(const void* x, int x_dt, long long ldx, const float* weight, void
   return dn_launch_status();
 }
 
+int dn_rmsnorm_add(const void* y, int y_dt, long long ldy, const float* weight, const float* scale, float mult, float* x, long long ldx,
+                   int T, int width, float eps, hipStream_t stream) {
+  if (!float_kind(y_dt)) return DN_ERR_DTYPE;
+  if (T < 0 || width < 1) return DN_ERR_SHAPE;
+  if (T == 0) return 0;
+  hipLaunchKernelGGL(rmsnorm_add_kernel, dim3(T), dim3(256), 0, stream, y, y_dt, static_cast<size_t>(ldy), weight, scale, mult, x,
+                     static_cast<size_t>(ldx), width, eps);
+  return dn_launch_status();
+}
+
+int dn_depth_mix(const float* hist, long long plane, int n, const float* w, float* out, long long total, hipStream_t stream) {
+  if (n < 1 || plane < total) return DN_ERR_SHAPE;
+  const int vec = plane % 4 == 0 && reinterpret_cast<uintptr_t>(hist) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0;
+  if (total == 0) return 0;
+  const long long groups = (total + 3) / 4;
+  hipLaunchKernelGGL(depth_mix_kernel, dim3(static_cast<unsigned>((groups + 255) / 256)), dim3(256), 0, stream, hist,
+                     static_cast<size_t>(plane), n, w, out, static_cast<size_t>(total), vec);
+  return dn_launch_status();
+}
+
+int dn_unit_heads(const float* x, long long ldx, float* out, long long ldo, int T, int H, int dim, float eps, float scale,
+                  hipStream_t stream) {
+  if (H < 1 || dim < 1) return DN_ERR_SHAPE;
+  if (T == 0) return 0;
+  hipLaunchKernelGGL(unit_heads_kernel, dim3(T, H), dim3(64), 0, stream, x, static_cast<size_t>(ldx), out, static_cast<size_t>(ldo), dim,
+                     eps, scale);
+  return dn_launch_status();
+}
+
 int dn_concat_cast(const float* a, long long lda, int wa, const float* b, long long ldb, int wb, void* out, int out_dt, int T,
                    hipStream_t stream) {
   if (!float_kind(out_dt)) return DN_ERR_DTYPE;
@@ -392,21 +530,23 @@ int dn_concat_cast(const float* a, long long lda, int wa, const float* b, long l
   return dn_launch_status();
 }
 
-int dn_conv_rows(const float* h, const float* w, const float* hist, const int* row_start, const int* slots, int S, int T, int width,
-                 int taps, void* out, int out_dt, long long hist_stride, hipStream_t stream) {
+int dn_conv_rows(const float* h, long long ldh, const float* w, const float* hist, const int* row_start, const int* slots, int S, int T,
+                 int width, int taps, int identity, int silu, void* out, int out_dt, long long ldo, long long hist_stride,
+                 hipStream_t stream) {
   if (!float_kind(out_dt)) return DN_ERR_DTYPE;
-  if (taps < 1 || S < 1) return DN_ERR_SHAPE;
+  if (taps < 1 || S < 1 || ldh < width || ldo < width) return DN_ERR_SHAPE;
   if (T == 0) return 0;
-  hipLaunchKernelGGL(conv_rows_kernel, dim3(T), dim3(256), 0, stream, h, w, hist, row_start, slots, S, width, taps, out, out_dt,
-                     static_cast<size_t>(hist_stride));
+  hipLaunchKernelGGL(conv_rows_kernel, dim3(T), dim3(256), 0, stream, h, static_cast<size_t>(ldh), w, hist, row_start, slots, S, width,
+                     taps, identity, silu, out, out_dt, static_cast<size_t>(ldo), static_cast<size_t>(hist_stride));
   return dn_launch_status();
 }
 
-int dn_history_update(const void* h, int h_dt, float* hist, const int* row_start, const int* slots, int S, int width, int keep,
-                      long long hist_stride, hipStream_t stream) {
+int dn_history_update(const void* h, int h_dt, long long ldh, float* hist, const int* row_start, const int* slots, int S, int width,
+                      int keep, long long hist_stride, hipStream_t stream) {
   if (!float_kind(h_dt)) return DN_ERR_DTYPE;
+  if (ldh < width) return DN_ERR_SHAPE;
   if (S == 0 || keep == 0) return 0;
-  hipLaunchKernelGGL(history_update_kernel, dim3(S), dim3(256), 0, stream, h, h_dt, hist, row_start, slots, width, keep,
+  hipLaunchKernelGGL(history_update_kernel, dim3(S), dim3(256), 0, stream, h, h_dt, static_cast<size_t>(ldh), hist, row_start, slots, width, keep,
                      static_cast<size_t>(hist_stride));
   return dn_launch_status();
 }
@@ -435,7 +575,7 @@ int dn_rotary(const void* src, int src_dt, long long ld_src, int src_off, int sr
 int dn_activate(const float* x, long long ldx, const float* bias, const float* lower, int kind, void* out, int out_dt, long long ldo,
                 int T, int n, hipStream_t stream) {
   if (!float_kind(out_dt)) return DN_ERR_DTYPE;
-  if (kind < 0 || kind > ACT_BOUNDED_SIGMOID) return DN_ERR_SHAPE;
+  if (kind < 0 || kind > ACT_XIELU || ((kind == ACT_XIELU || kind == ACT_EXP_NEG_SOFTPLUS) && !lower)) return DN_ERR_SHAPE;
   if (T == 0) return 0;
   hipLaunchKernelGGL(activate_kernel, dim3(T), dim3(256), 0, stream, x, static_cast<size_t>(ldx), bias, lower, kind, out, out_dt,
                      static_cast<size_t>(ldo), n);
@@ -453,19 +593,23 @@ int dn_gated(const void* x, int x_dt, long long ldx, const float* g, long long l
 }
 
 int dn_state_scan(const float* r, long long ldr, const float* k, long long ldk, const float* v, long long ldv, const float* w,
-                  long long ldw, const float* u, float* state, long long slot_stride, const int* row_start, const int* slots, int S,
-                  int T, int H, int dk, int dv, int read_after, int key_from_decay, float* out, long long ldo, hipStream_t stream) {
-  if (dk < 1 || dk > 256 || dv < 1 || H < 1) return DN_ERR_SHAPE;
+                  long long ldw, const float* u, const float* beta, long long ldb, const float* w_head, int G, float* state,
+                  long long slot_stride, const int* row_start, const int* slots, int S, int T, int H, int dk, int dv, int mode,
+                  int key_from_decay, float* out, long long ldo, hipStream_t stream) {
+  if (dk < 1 || dk > 256 || dv < 1 || H < 1 || G < 1 || H % G != 0) return DN_ERR_SHAPE;
   if (!key_from_decay && k == nullptr) return DN_ERR_SHAPE;
+  if (mode < SCAN_BEFORE || mode > SCAN_DELTA || (mode == SCAN_DELTA && beta == nullptr) || (w == nullptr) == (w_head == nullptr))
+    return DN_ERR_SHAPE;
   if (S == 0) return 0;
-  ScanArgs a{r, k, v, w, u, static_cast<size_t>(ldr), static_cast<size_t>(ldk), static_cast<size_t>(ldv), static_cast<size_t>(ldw),
-             state, static_cast<size_t>(slot_stride), row_start, slots, H, dk, dv, read_after, key_from_decay, out,
+  const int read_after = mode;
+  ScanArgs a{r, k, v, w, u, beta, w_head, static_cast<size_t>(ldr), static_cast<size_t>(ldk), static_cast<size_t>(ldv),
+             static_cast<size_t>(ldw), static_cast<size_t>(ldb), G, state, static_cast<size_t>(slot_stride), row_start, slots, H, dk, dv, read_after, key_from_decay, out,
              static_cast<size_t>(ldo)};
   // (the parts of a column's sum by the head's size alone, never by the step: a row's bits are the same in every step)
   const dim3 few((dv + 15) / 16, H, S), many((dv + 3) / 4, H, S);
   auto by16 = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
-  const bool vec = dk % 4 == 0 && dv % 4 == 0 && ldr % 4 == 0 && ldv % 4 == 0 && ldw % 4 == 0 && (key_from_decay || ldk % 4 == 0) &&
-                   by16(r) && by16(v) && by16(w) && (key_from_decay || by16(k));
+  const bool vec = dk % 4 == 0 && dv % 4 == 0 && ldr % 4 == 0 && ldv % 4 == 0 && (w == nullptr || ldw % 4 == 0) &&
+                   (key_from_decay || ldk % 4 == 0) && by16(r) && by16(v) && by16(w) && (key_from_decay || by16(k));
   const bool few_rows = T <= 2 * S;      // (decoded tokens: a row or two a request)
 #define DN_SCAN3(DK, KG, GRID, AFTER, VEC)                                                                    \
   do {                                                                                                        \
@@ -477,10 +621,11 @@ int dn_state_scan(const float* r, long long ldr, const float* k, long long ldk, 
     if (vec) DN_SCAN3(DK, KG, GRID, AFTER, true); \
     else DN_SCAN3(DK, KG, GRID, AFTER, false);    \
   } while (0)
-#define DN_SCAN(DK, KG, GRID)                \
-  do {                                       \
-    if (read_after) DN_SCAN2(DK, KG, GRID, true); \
-    else DN_SCAN2(DK, KG, GRID, false);      \
+#define DN_SCAN(DK, KG, GRID)                                     \
+  do {                                                            \
+    if (mode == SCAN_DELTA) DN_SCAN2(DK, KG, GRID, SCAN_DELTA);   \
+    else if (mode == SCAN_AFTER) DN_SCAN2(DK, KG, GRID, SCAN_AFTER); \
+    else DN_SCAN2(DK, KG, GRID, SCAN_BEFORE);                     \
   } while (0)
   if (dk <= 16) DN_SCAN(16, 4, few);
   else if (dk <= 32) DN_SCAN(32, 4, few);

@@ -125,21 +125,24 @@ def _declare(name, lib):
         "sequence": {
             "dn_rmsnorm": [P, I, c_longlong, P, P, I, c_longlong, P, I, I, F, P],
             "dn_concat_cast": [P, c_longlong, I, P, c_longlong, I, P, I, I, P],
-            "dn_conv_rows": [P, P, P, P, P, I, I, I, I, P, I, c_longlong, P],
-            "dn_history_update": [P, I, P, P, P, I, I, I, c_longlong, P],
+            "dn_rmsnorm_add": [P, I, c_longlong, P, P, F, P, c_longlong, I, I, F, P],
+            "dn_depth_mix": [P, c_longlong, I, P, P, c_longlong, P],
+            "dn_unit_heads": [P, c_longlong, P, c_longlong, I, I, I, F, F, P],
+            "dn_conv_rows": [P, c_longlong, P, P, P, P, I, I, I, I, I, I, P, I, c_longlong, c_longlong, P],
+            "dn_history_update": [P, I, c_longlong, P, P, P, I, I, I, c_longlong, P],
             "dn_shift_mix": [P, I, P, P, I, P, P, I, I, I, P, I, c_longlong, P],
             "dn_rotary": [P, I, c_longlong, I, I, P, I, c_longlong, I, I, P, P, I, I, I, I, P],
             "dn_activate": [P, c_longlong, P, P, I, P, I, c_longlong, I, I, P],
             "dn_gated": [P, I, c_longlong, P, c_longlong, I, P, I, c_longlong, I, I, P],
-            "dn_state_scan": [P, c_longlong, P, c_longlong, P, c_longlong, P, c_longlong, P, P, c_longlong, P, P, I, I, I, I, I, I, I,
-                              P, c_longlong, P],
+            "dn_state_scan": [P, c_longlong, P, c_longlong, P, c_longlong, P, c_longlong, P, P, c_longlong, P, I, P, c_longlong, P, P,
+                              I, I, I, I, I, I, I, P, c_longlong, P],
             "dn_head_norm": [P, c_longlong, P, I, F, P, c_longlong, I, P, I, c_longlong, I, I, I, P],
         },
         "grouped": {
             "dn_heads_linear": [P, I, c_longlong, I, I, P, I, P, I, c_longlong, I, I, I, I, I, I, P],
-            "dn_moe_route": [P, P, I, I, I, P, P, P],
+            "dn_moe_route": [P, c_longlong, P, I, I, I, I, I, P, P, P],
             "dn_moe_plan": [P, I, I, P, P, P],
-            "dn_moe_up": [P, I, c_longlong, P, P, I, I, I, P, P, I, I, I, F, F, P, I, I, P],
+            "dn_moe_up": [P, I, c_longlong, P, P, I, I, I, P, P, I, I, I, F, F, I, P, P, I, I, P],
             "dn_moe_down": [P, I, P, P, I, I, P, I, I, I, P, I, P],
             "dn_moe_combine": [P, P, I, I, I, P, c_longlong, P],
         },
@@ -910,7 +913,7 @@ def linear_norm_in(copy, stats, c1, c2, eps, w, out, epilogue="none", kv=None, n
 
 
 # -- layers that carry more than keys and values from token to token (csrc/kernels/sequence.hip) -----------------------
-ACTIVATIONS = {"silu": 0, "sigmoid": 1, "tanh": 2, "exp_neg_exp": 3, "bounded_sigmoid": 4}
+ACTIVATIONS = {"silu": 0, "sigmoid": 1, "tanh": 2, "exp_neg_exp": 3, "bounded_sigmoid": 4, "exp_neg_softplus": 5, "xielu": 6}
 
 
 def _f32vec(t, name, n=None):
@@ -953,6 +956,43 @@ def rmsnorm(x, weight, eps, out, rows=None):
     return out
 
 
+def rmsnorm_add(y, weight, scale, mult, eps, x):
+    """x[t, :] += mult * (y[t, :] / sqrt(mean(y[t, :]^2) + eps) * weight) * scale; weight and scale: 32-bit vectors or None;
+    x: 32-bit rows (the stream), changed in place; statistics in 32-bit."""
+    _dev(y, "y", _FLOATS, 2), _dev(x, "x", (torch.float32,), 2)
+    T, width = y.shape
+    _need(tuple(x.shape) == (T, width), "rmsnorm_add: shapes")
+    _f32vec(weight, "weight", width), _f32vec(scale, "scale", width)
+    _ok(_lib("sequence").dn_rmsnorm_add(y.data_ptr(), _CODE[y.dtype], _rows(y, "y"), _ptr(weight), _ptr(scale), float(mult),
+                                        x.data_ptr(), _rows(x, "x"), T, width, float(eps), _stream()), "rmsnorm_add")
+    return x
+
+
+def depth_mix(hist, n, weights, out):
+    """out = sum over j < n of weights[j] * hist[j], j ascending; hist: 32-bit [planes, rows, width], contiguous; weights:
+    at least n 32-bit numbers; out: 32-bit [rows, width], contiguous; it may be a plane of hist from n on."""
+    _dev(hist, "hist", (torch.float32,), 3), _dev(out, "out", (torch.float32,), 2)
+    _f32vec(weights, "weights")
+    planes, T, width = hist.shape
+    _need(hist.is_contiguous() and out.is_contiguous() and tuple(out.shape) == (T, width) and 1 <= n <= planes
+          and weights.numel() >= n, "depth_mix: shapes")
+    _ok(_lib("sequence").dn_depth_mix(hist.data_ptr(), T * width, n, weights.data_ptr(), out.data_ptr(), T * width, _stream()),
+        "depth_mix")
+    return out
+
+
+def unit_heads(x, n_heads, dim, eps, scale, out):
+    """out[t, h, :] = x[t, h, :] / sqrt(sum(x[t, h, :]^2) + eps) * scale for the n_heads vectors of `dim` numbers at the start
+    of each row; x and out 32-bit (out may be x)."""
+    _dev(x, "x", (torch.float32,), 2), _dev(out, "out", (torch.float32,), 2)
+    T = x.shape[0]
+    _need(out.shape[0] == T and x.shape[1] >= n_heads * dim and out.shape[1] >= n_heads * dim and n_heads >= 1 and dim >= 1,
+          "unit_heads: shapes")
+    _ok(_lib("sequence").dn_unit_heads(x.data_ptr(), _rows(x, "x"), out.data_ptr(), _rows(out, "out"), T, n_heads, dim, float(eps),
+                                       float(scale), _stream()), "unit_heads")
+    return out
+
+
 def concat_cast(a, b, out):
     """out[t, :] = [a[t, :] | b[t, :]], a and b 32-bit, out contiguous in its own dtype."""
     _dev(a, "a", (torch.float32,), 2), _dev(b, "b", (torch.float32,), 2), _dev(out, "out", _FLOATS, 2)
@@ -963,33 +1003,35 @@ def concat_cast(a, b, out):
     return out
 
 
-def conv_rows(h, w, hist, row_start, slots, out):
-    """out[t, c] = h[t, c] + sum_j w[c, j] h[t - taps + 1 + j, c] inside each request; the rows before a request's first
-    row of this step come from hist [slots, (taps - 1) * width] (oldest first).  h 32-bit [T, width]."""
+def conv_rows(h, w, hist, row_start, slots, out, identity=True, act=None):
+    """out[t, c] = act((h[t, c] if identity else 0) + sum_j w[c, j] h[t - taps + 1 + j, c]) inside each request; the rows
+    before a request's first row of this step come from hist [slots, (taps - 1) * width] (oldest first).  h: 32-bit rows whose
+    first `width` columns are the channels (width = w.shape[0]); act: None or "silu"."""
     _dev(h, "h", (torch.float32,), 2), _dev(w, "w", (torch.float32,), 2), _dev(out, "out", _FLOATS, 2)
-    T, width = h.shape
-    taps = w.shape[1]
+    T = h.shape[0]
+    width, taps = w.shape
     S = _request_tables(row_start, slots, "conv_rows")
-    _need(h.is_contiguous() and out.is_contiguous() and w.is_contiguous() and w.shape[0] == width and tuple(out.shape) == (T, width),
-          "conv_rows: shapes")
+    _need(h.shape[1] >= width and w.is_contiguous() and tuple(out.shape) == (T, width) and act in (None, "silu"), "conv_rows: shapes")
     stride = _history(hist, (taps - 1) * width, "conv_rows") if taps > 1 else 0
-    _ok(_lib("sequence").dn_conv_rows(h.data_ptr(), w.data_ptr(), _ptr(hist) if taps > 1 else 0, row_start.data_ptr(),
-                                      slots.data_ptr(), S, T, width, taps, out.data_ptr(), _CODE[out.dtype], stride, _stream()),
+    _ok(_lib("sequence").dn_conv_rows(h.data_ptr(), _rows(h, "h"), w.data_ptr(), _ptr(hist) if taps > 1 else 0, row_start.data_ptr(),
+                                      slots.data_ptr(), S, T, width, taps, int(bool(identity)), int(act == "silu"), out.data_ptr(),
+                                      _CODE[out.dtype], _rows(out, "out"), stride, _stream()),
         "conv_rows")
     return out
 
 
 def history_update(h, hist, row_start, slots):
-    """hist [slots, keep * width]: the last `keep` rows of (a request's history ++ its rows of this step) become its history."""
+    """hist [slots, keep * width]: the last `keep` rows of (a request's history ++ its rows of this step) become its history;
+    width = h.shape[1] (h may be the first columns of wider rows)."""
     _dev(h, "h", _FLOATS, 2)
     T, width = h.shape
     S = _request_tables(row_start, slots, "history_update")
     _dev(hist, "history", (torch.float32,), 2)
-    _need(h.is_contiguous() and hist.shape[1] % width == 0, "history_update: shapes")
+    _need(hist.shape[1] % width == 0, "history_update: shapes")
     keep = hist.shape[1] // width
     stride = _history(hist, keep * width, "history_update")
-    _ok(_lib("sequence").dn_history_update(h.data_ptr(), _CODE[h.dtype], hist.data_ptr(), row_start.data_ptr(), slots.data_ptr(),
-                                           S, width, keep, stride, _stream()), "history_update")
+    _ok(_lib("sequence").dn_history_update(h.data_ptr(), _CODE[h.dtype], _rows(h, "h"), hist.data_ptr(), row_start.data_ptr(),
+                                           slots.data_ptr(), S, width, keep, stride, _stream()), "history_update")
 
 
 def shift_mix(h, hist, mu, row_start, slots, out):
@@ -1028,11 +1070,13 @@ def rotary(src, dst, positions, freq, n_vec, dims, width, src_off=0, src_stride=
 
 def activate(x, kind, out, bias=None, lower=None):
     """out = act(x + bias): "silu", "sigmoid", "tanh", "exp_neg_exp" (exp(-exp(z))), "bounded_sigmoid"
-    (lower + (1 - lower) * sigmoid(z)).  x 32-bit; out may be x."""
+    (lower + (1 - lower) * sigmoid(z)), "exp_neg_softplus" (exp(-lower * log(1 + e^z)), lower a rate per column), "xielu"
+    (z > 0: a z^2 + z / 2, else b (e^z - 1 - z) + z / 2, with lower = (a, b), two numbers).  x 32-bit; out may be x."""
     _dev(x, "x", (torch.float32,), 2), _dev(out, "out", _FLOATS, 2)
     T, n = x.shape
     _need(tuple(out.shape) == (T, n), "activate: shapes")
-    _f32vec(bias, "bias", n), _f32vec(lower, "lower", n)
+    _need(kind not in ("xielu", "exp_neg_softplus") or lower is not None, lambda: f"activate: {kind} needs its numbers in `lower`")
+    _f32vec(bias, "bias", n), _f32vec(lower, "lower", 2 if kind == "xielu" else n)
     _ok(_lib("sequence").dn_activate(x.data_ptr(), _rows(x, "x"), _ptr(bias), _ptr(lower), ACTIVATIONS[kind], out.data_ptr(),
                                      _CODE[out.dtype], _rows(out, "out"), T, n, _stream()), "activate")
     return out
@@ -1048,27 +1092,40 @@ def gated(x, g, kind, out):
     return out
 
 
-def state_scan(r, k, v, w, u, state, row_start, slots, n_heads, dk, dv, out, read_after=False, key_from_decay=False):
+def state_scan(r, k, v, w, u, state, row_start, slots, n_heads, dk, dv, out, read_after=False, key_from_decay=False, beta=None,
+               w_head=None, qk_heads=None):
     """The recurrence of a matrix state per head, S [dk, dv], over each request's rows of this step in order:
       a = 1 - w if key_from_decay else k
       read_after:  S <- diag(w) S + a v^T ;  o = S^T r
+      beta given:  S <- diag(w) S ;  e = beta (v - S^T a) ;  S <- S + a e^T ;  o = S^T r        (the delta rule)
       else:        o = (S + diag(u) a v^T)^T r ;  S <- diag(w) S + a v^T        (u None: no bonus)
-    r, k, w: 32-bit [T, heads * dk]; v, out: 32-bit [T, heads * dv]; state: 32-bit [slots, heads * dv * dk] (a head's state
+    r, k: 32-bit [T, qk_heads * dk] (qk_heads None: n_heads; fewer: head h reads head h // (n_heads // qk_heads));
+    w: 32-bit [T, heads * dk], or None with w_head: 32-bit [heads], one decay per head for every row and channel;
+    v, out: 32-bit [T, heads * dv]; beta: 32-bit [T, heads]; state: 32-bit [slots, heads * dv * dk] (a head's state
     held [value column][key channel]), read and written at the requests' slots."""
-    for t, name, n in ((r, "r", dk), (w, "w", dk), (v, "v", dv), (out, "out", dv)) + (() if key_from_decay else ((k, "k", dk),)):
+    G = n_heads if qk_heads is None else qk_heads
+    _need(G >= 1 and n_heads % G == 0, lambda: f"state_scan: {n_heads} heads over {G} heads of queries and keys")
+    _need((w is None) != (w_head is None), "state_scan: a decay per row and channel (w) or one per head (w_head)")
+    _need(not (key_from_decay and w is None), "state_scan: keys from the decay need w")
+    given = ((r, "r", G * dk), (v, "v", n_heads * dv), (out, "out", n_heads * dv)) + (() if key_from_decay else ((k, "k", G * dk),)) \
+        + (() if w is None else ((w, "w", n_heads * dk),)) + (() if beta is None else ((beta, "beta", n_heads),))
+    for t, name, n in given:
         _dev(t, name, (torch.float32,), 2)
-        _need(t.shape[1] == n_heads * n, lambda: f"state_scan: {name} {tuple(t.shape)}")
+        _need(t.shape[1] == n, lambda: f"state_scan: {name} {tuple(t.shape)}")
     T = r.shape[0]
     S = _request_tables(row_start, slots, "state_scan")
-    _need(all(t.shape[0] == T for t in (v, w, out)), "state_scan: rows")
+    _need(all(t.shape[0] == T for t, _, _ in given), "state_scan: rows")
     _need(1 <= dk <= 256, lambda: f"state_scan: {dk} key channels a head; the kernel keeps up to 256 in registers")
-    _f32vec(u, "u", n_heads * dk)
+    _need(beta is None or (not read_after and u is None), "state_scan: the delta rule reads after its write and has no bonus")
+    _f32vec(u, "u", n_heads * dk), _f32vec(w_head, "w_head", n_heads)
     stride = _history(state, n_heads * dk * dv, "state_scan")
+    mode = 2 if beta is not None else int(bool(read_after))
     _ok(_lib("sequence").dn_state_scan(r.data_ptr(), _rows(r, "r"), 0 if key_from_decay else k.data_ptr(),
-                                       0 if key_from_decay else _rows(k, "k"), v.data_ptr(), _rows(v, "v"), w.data_ptr(),
-                                       _rows(w, "w"), _ptr(u), state.data_ptr(), stride, row_start.data_ptr(), slots.data_ptr(), S,
-                                       T, n_heads, dk, dv, int(read_after), int(key_from_decay), out.data_ptr(), _rows(out, "out"),
-                                       _stream()), "state_scan")
+                                       0 if key_from_decay else _rows(k, "k"), v.data_ptr(), _rows(v, "v"), _ptr(w),
+                                       _rows(w, "w") if w is not None else 0, _ptr(u), _ptr(beta),
+                                       _rows(beta, "beta") if beta is not None else 0, _ptr(w_head), G, state.data_ptr(), stride,
+                                       row_start.data_ptr(), slots.data_ptr(), S, T, n_heads, dk, dv, mode, int(key_from_decay),
+                                       out.data_ptr(), _rows(out, "out"), _stream()), "state_scan")
     return out
 
 
@@ -1110,15 +1167,19 @@ def heads_linear(a, w, out, a_off=0, a_stride=None, o_off=0, o_stride=None):
     return out
 
 
-def moe_route(z, correction, top, ids, wts):
-    """Per row: s = softmax(z); the `top` experts with the largest s + correction (the lower index wins a tie) go to ids
-    [T, top], their s divided by the sum of the chosen s (+ 1e-20) to wts [T, top]."""
+def moe_route(z, correction, top, ids, wts, score="softmax", renorm=True, n_experts=None):
+    """Per row: s = softmax(z) over the experts, or (score "sigmoid") each expert's own 1 / (1 + e^-z); the `top` experts with
+    the largest s + correction (the lower index wins a tie) go to ids [T, top]; wts [T, top] gets their s divided by the sum
+    of the chosen s (+ 1e-20), or (renorm False) their s as it is.  n_experts: the first columns of z that are experts
+    (None: all of them)."""
     _dev(z, "z", (torch.float32,), 2), _dev(ids, "ids", _I32, 2), _dev(wts, "wts", (torch.float32,), 2)
-    T, E = z.shape
-    _need(z.is_contiguous() and ids.is_contiguous() and wts.is_contiguous() and tuple(ids.shape) == (T, top)
-          and tuple(wts.shape) == (T, top) and 1 <= top <= E, "moe_route: shapes")
+    T = z.shape[0]
+    E = z.shape[1] if n_experts is None else n_experts
+    _need(ids.is_contiguous() and wts.is_contiguous() and tuple(ids.shape) == (T, top) and E <= z.shape[1]
+          and tuple(wts.shape) == (T, top) and 1 <= top <= E and score in ("softmax", "sigmoid"), "moe_route: shapes")
     _f32vec(correction, "correction", E)
-    _ok(_lib("grouped").dn_moe_route(z.data_ptr(), _ptr(correction), T, E, top, ids.data_ptr(), wts.data_ptr(), _stream()), "moe_route")
+    _ok(_lib("grouped").dn_moe_route(z.data_ptr(), _rows(z, "z"), _ptr(correction), T, E, top, int(score == "sigmoid"),
+                                     int(bool(renorm)), ids.data_ptr(), wts.data_ptr(), _stream()), "moe_route")
 
 
 def moe_plan(ids, n_experts, offsets, order):
@@ -1137,9 +1198,11 @@ def experts_packable(n_experts, rows, inner):
     return rows % 16 == 0 and inner % 32 == 0
 
 
-def moe_up(h, order, offsets, top, w_gate, w_up, limit, alpha, y, dims=None):
-    """For place p of expert e, the row t = order[p] // top: g = min(w_gate[e] h[t], limit), u = clamp(w_up[e] h[t], -limit,
-    limit), y[p] = g * sigmoid(alpha * g) * (u + 1).  w_gate, w_up: [experts, ff, width]; y [T * top, ff].
+def moe_up(h, order, offsets, top, w_gate, w_up, limit, alpha, y, dims=None, kind="clamped", in_scale=None):
+    """For place p of expert e, the row t = order[p] // top: kind "clamped": g = min(w_gate[e] h[t], limit), u = clamp(w_up[e]
+    h[t], -limit, limit), y[p] = g * sigmoid(alpha * g) * (u + 1); kind "silu": the expert reads s h[t] with s =
+    in_scale[order[p]] (32-bit [T * top]; None: 1), y[p] = silu(w_gate[e] s h[t]) * (w_up[e] s h[t]), the factor applied to
+    the 32-bit sums.  w_gate, w_up: [experts, ff, width]; y [T * top, ff].
     dims = (experts, ff, width): w_gate and w_up are PackedMatrix of the stacked [experts * ff, width] (experts_packable)."""
     _dev(h, "h", _FLOATS, 2), _dev(y, "y", _FLOATS, 2)
     n = order.shape[0]
@@ -1154,10 +1217,14 @@ def moe_up(h, order, offsets, top, w_gate, w_up, limit, alpha, y, dims=None):
         _need(w_gate.is_contiguous() and w_up.is_contiguous() and tuple(w_up.shape) == (E, ff, width), "moe_up: weights")
         wdt = w_gate.dtype
     _need(h.shape[1] == width and y.is_contiguous() and tuple(y.shape) == (n, ff) and offsets.shape[0] == E + 1
-          and n == h.shape[0] * top, "moe_up: shapes")
+          and n == h.shape[0] * top and kind in ("clamped", "silu"), "moe_up: shapes")
+    if in_scale is not None:
+        _dev(in_scale, "in_scale", (torch.float32,))
+        _need(in_scale.is_contiguous() and in_scale.numel() == n and kind == "silu", "moe_up: in_scale")
     _ok(_lib("grouped").dn_moe_up(h.data_ptr(), _CODE[h.dtype], _rows(h, "h"), order.data_ptr(), offsets.data_ptr(), E, top, n,
                                   w_gate.data_ptr(), w_up.data_ptr(), _CODE[wdt], ff, width, float(limit), float(alpha),
-                                  y.data_ptr(), _CODE[y.dtype], int(dims is not None), _stream()), "moe_up")
+                                  int(kind == "silu"), _ptr(in_scale), y.data_ptr(), _CODE[y.dtype], int(dims is not None),
+                                  _stream()), "moe_up")
 
 
 def moe_down(y, order, offsets, w_down, out, dims=None):
@@ -1182,10 +1249,13 @@ def moe_down(y, order, offsets, w_down, out, dims=None):
 
 
 def moe_combine(out, wts, x):
-    """x[t, :] += sum_c wts[t, c] * out[t * top + c, :], the choices in their order."""
-    _dev(out, "out", (torch.float32,), 2), _dev(wts, "wts", (torch.float32,), 2), _dev(x, "x", (torch.float32,), 2)
-    T, top = wts.shape
-    width = x.shape[1]
-    _need(out.is_contiguous() and wts.is_contiguous() and tuple(out.shape) == (T * top, width) and x.shape[0] == T, "moe_combine: shapes")
-    _ok(_lib("grouped").dn_moe_combine(out.data_ptr(), wts.data_ptr(), T, top, width, x.data_ptr(), _rows(x, "x"), _stream()),
+    """x[t, :] += sum_c wts[t, c] * out[t * top + c, :], the choices in their order (wts None: every weight is 1)."""
+    _dev(out, "out", (torch.float32,), 2), _dev(x, "x", (torch.float32,), 2)
+    T, width = x.shape
+    top = out.shape[0] // max(T, 1) if wts is None else wts.shape[1]
+    if wts is not None:
+        _dev(wts, "wts", (torch.float32,), 2)
+        _need(wts.is_contiguous() and wts.shape[0] == T, "moe_combine: weights")
+    _need(out.is_contiguous() and tuple(out.shape) == (T * top, width), "moe_combine: shapes")
+    _ok(_lib("grouped").dn_moe_combine(out.data_ptr(), _ptr(wts), T, top, width, x.data_ptr(), _rows(x, "x"), _stream()),
         "moe_combine")

@@ -8,6 +8,8 @@ caches) and runs them (`forward(x, ctx, caches, runtime)`, `caches` in that same
 from __future__ import annotations
 
 from ..kernels import ops
+import torch
+
 from .base import ARRANGEMENTS, DeferredSum, LazyNorm, StreamStats
 
 
@@ -115,3 +117,43 @@ class FilteredPreNormBlock:
         self.mixer.forward(h, ctx, caches[1], accumulate_into=x)
         if self.has_ffn:
             self.ffn.forward(self.norm2.forward(x, runtime.act_dtype), ctx, accumulate_into=x)
+
+
+@ARRANGEMENTS.register("sandwich")
+class SandwichBlock:
+    """A norm before and a norm behind each sublayer: x += post1(mixer(norm1(x))); x += post2(ffn(norm2(x))).  The norms
+    behind are of a kind that adds into the stream itself (`add_into(y, x)`, parts.norms.StreamRMSNorm: a multiplier of
+    the model and a vector of the layer ride along).  A block whose feed-forward is "none" ends after the mixer."""
+
+    SLOTS = {"norm1": "norm", "mixer": "mixer", "post1": "norm", "norm2": "norm", "ffn": "feed_forward", "post2": "norm"}
+
+    def __init__(self, norm1, mixer, post1, norm2, ffn, post2):
+        self.norm1, self.mixer, self.post1, self.norm2, self.ffn, self.post2 = norm1, mixer, post1, norm2, ffn, post2
+        self.has_ffn = not getattr(ffn, "absent", False)
+        for n in (post1, post2):
+            if not hasattr(n, "add_into"):
+                raise TypeError(f"sandwich: the norm behind a sublayer must add into the stream; {type(n).__name__} does not")
+
+    def parts(self):
+        return [self.norm1, self.mixer, self.post1] + ([self.norm2, self.ffn, self.post2] if self.has_ffn else [])
+
+    def mixers(self):
+        return [self.mixer]
+
+    @staticmethod
+    def _result(part, x, *args):
+        """The sublayer's result as 32-bit rows of its own: from a part that can return them (`returns_rows`), or
+        added by the part into rows of zeros."""
+        if getattr(part, "returns_rows", False):
+            return part.forward(*args, accumulate_into=None)
+        y = torch.zeros(x.shape, dtype=torch.float32, device=x.device)
+        part.forward(*args, accumulate_into=y)
+        return y
+
+    def forward(self, x, ctx, caches, runtime):
+        runtime.stream_stats = None
+        h = self.norm1.forward(x, runtime.act_dtype)
+        self.post1.add_into(self._result(self.mixer, x, h, ctx, caches[0]), x)
+        if self.has_ffn:
+            h = self.norm2.forward(x, runtime.act_dtype)
+            self.post2.add_into(self._result(self.ffn, x, h, ctx), x)

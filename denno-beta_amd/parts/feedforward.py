@@ -9,33 +9,50 @@ from .base import FEED_FORWARDS, Part
 from .linear import Linear
 
 ACTIVATION_EPILOGUES = {"gelu_tanh": "gelu_tanh", "gelu_erf": "gelu_erf"}
+# activations with numbers of their own in a tensor: a kernel between the two products, on the first one's 32-bit result
+ACTIVATION_KERNELS = ("xielu",)
+F32 = torch.float32
 
 
 @FEED_FORWARDS.register("dense_mlp")
 class DenseMLP(Part):
     """act(h W_up + b_up) W_down + b_down, added into the residual stream
     (crates/denno-engine/src/model/gpt2.rs:211-219).  The activation runs in the first
-    product's epilogue, in 32-bit, before the rounding to the activation dtype."""
+    product's epilogue, in 32-bit, before the rounding to the activation dtype.
+
+    activation "xielu": z > 0: softplus(p) z^2 + z / 2; else (1/2 + softplus(q)) (e^z - 1 - z) + z / 2, with (p, q) the two
+    numbers of the tensor `activation_params`; it runs as a kernel of its own on the first product's 32-bit result."""
     graph_safe = True
+    returns_rows = True
 
     def __init__(self, width: int, inner: int, activation: str, up_weight: str, up_bias, down_weight: str,
-                 down_bias, stored_in_out: bool = False, down_init_std: float = 0.02):
-        if activation not in ACTIVATION_EPILOGUES:
-            raise ValueError(f"activation {activation!r}; known: {sorted(ACTIVATION_EPILOGUES)}")
-        self.width, self.inner, self.activation = width, inner, activation
+                 down_bias, stored_in_out: bool = False, down_init_std: float = 0.02, activation_params=None):
+        if activation not in ACTIVATION_EPILOGUES and activation not in ACTIVATION_KERNELS:
+            raise ValueError(f"activation {activation!r}; known: {sorted(ACTIVATION_EPILOGUES) + list(ACTIVATION_KERNELS)}")
+        if (activation in ACTIVATION_KERNELS) != (activation_params is not None):
+            raise ValueError(f"activation {activation!r}: the tensor of its numbers is " +
+                             ("missing" if activation_params is None else "not used"))
+        self.width, self.inner, self.activation, self.activation_params = width, inner, activation, activation_params
+        if activation in ACTIVATION_KERNELS:
+            self.libraries = ("sequence",)
         self.up = Linear(width, inner, up_weight, up_bias, stored_in_out)
         self.down = Linear(inner, width, down_weight, down_bias, stored_in_out, down_init_std)
 
     def param_specs(self):
-        return self.up.param_specs() + self.down.param_specs()
+        own = [ParamSpec(self.activation_params, (2,), "vector", ("normal", 0.3, 0.3))] if self.activation_params else []
+        return self.up.param_specs() + self.down.param_specs() + own
 
     def bind(self, tensors, runtime):
         super().bind(tensors, runtime)
         self.up.bind(tensors)
         self.down.bind(tensors)
+        if self.activation_params:
+            pq = tensors[self.activation_params].to(F32)
+            sp = torch.nn.functional.softplus(pq)
+            self.act_numbers = torch.stack([sp[0], 0.5 + sp[1]]).contiguous()      # (softplus(p), 1/2 + softplus(q)), once
 
     def packed_input(self, n_rows):
-        return self.up.packed_input(n_rows)
+        return self.activation in ACTIVATION_EPILOGUES and self.up.packed_input(n_rows)
 
     def prepare_lazy_norm(self, norm):
         self.up.fold_norm(norm)
@@ -51,8 +68,15 @@ class DenseMLP(Part):
 
     def forward(self, h, ctx, accumulate_into, stats=None, deferred=None):
         n = h.shape[0]
-        f = self.up(h, out_dtype=self.runtime.act_dtype, epilogue=ACTIVATION_EPILOGUES[self.activation],
-                    packed_out=self.up.few_rows(n) and self.down.packed_input(n))
+        if self.activation in ACTIVATION_KERNELS:
+            z = self.up(h, out_dtype=F32)
+            f = ops.activate(z, self.activation, torch.empty(z.shape, dtype=self.runtime.act_dtype, device=z.device),
+                             lower=self.act_numbers)
+        else:
+            f = self.up(h, out_dtype=self.runtime.act_dtype, epilogue=ACTIVATION_EPILOGUES[self.activation],
+                        packed_out=self.up.few_rows(n) and self.down.packed_input(n) and accumulate_into is not None)
+        if accumulate_into is None:
+            return self.down(f, out_dtype=F32)
         self.down(f, residual=accumulate_into, stats=stats, deferred=deferred)
 
 
@@ -75,20 +99,44 @@ class RoutedExperts(Part):
     token's `top` experts are the ones with the largest s + correction, its weights their s divided by their sum
     (+ 1e-20).  An expert: g = min(W_gate h, limit), u = clamp(W_up h, -limit, limit), W_down (g sigmoid(alpha g) (u + 1)).
     The step's (token, expert) pairs are sorted by expert on the device, each expert's products run over tiles of its
-    own rows, and the results are added into the stream per token in the order of its choices."""
-    graph_safe = True
-    libraries = ("grouped",)
+    own rows, and the results are added into the stream per token in the order of its choices.
 
-    def __init__(self, width: int, inner: int, n_experts: int, top: int, limit: float, alpha: float, router: str,
-                 correction, gate: str, up: str, down: str):
+    What an architecture may choose otherwise: score "sigmoid" (each expert's own 1 / (1 + e^-z)); renorm False (the
+    weights are the chosen scores as they are); weigh "input" (a weight multiplies what the expert reads, not what it
+    returns); act "silu" (an expert is W_down (silu(W_gate h) * (W_up h)), nothing clamped; limit and alpha are then not
+    used); shared: an expert of the same form that every token uses, dict(inner, gate, up, down, token_gate): its result is
+    added, times sigmoid(w . h) with w the vector `token_gate` (a name, or None: as it is)."""
+    graph_safe = True
+    returns_rows = True
+    libraries = ("grouped", "sequence")
+
+    def __init__(self, width: int, inner: int, n_experts: int, top: int, router: str, correction, gate: str, up: str, down: str,
+                 limit: float = 0.0, alpha: float = 1.0, score: str = "softmax", renorm: bool = True, weigh: str = "output",
+                 act: str = "clamped", shared=None):
         """gate, up, down: tensor names with {e} for the expert's number; correction: a name or None."""
         if not 1 <= top <= n_experts:
             raise ValueError(f"routed_experts: {top} of {n_experts} experts")
+        if score not in ("softmax", "sigmoid") or weigh not in ("output", "input") or act not in ("clamped", "silu"):
+            raise ValueError(f"routed_experts: score {score!r}, weigh {weigh!r}, act {act!r}")
+        if weigh == "input" and act != "silu":
+            raise ValueError("routed_experts: a weight on what the expert reads goes with act 'silu'")
         self.width, self.inner, self.n_experts, self.top = width, inner, n_experts, top
         self.limit, self.alpha = float(limit), float(alpha)
-        self.router = Linear(width, n_experts, router, None)
+        self.score, self.renorm, self.weigh, self.act = score, bool(renorm), weigh, act
         self.correction_name = correction
         self.templates = dict(gate=gate, up=up, down=down)
+        self.shared = dict(shared) if shared else None
+        self.token_gate = self.shared.get("token_gate") if self.shared else None
+        # the router, and behind its rows the shared expert's gate: one product for both
+        if self.token_gate:
+            self.router = Linear(width, n_experts + 1, router + "+gate", None, weight_sources=((router, n_experts), (self.token_gate, 1)))
+        else:
+            self.router = Linear(width, n_experts, router, None)
+        if self.shared:
+            sh = self.shared
+            self.shared_up = Linear(width, 2 * sh["inner"], sh["gate"] + "+up", None,
+                                    weight_sources=((sh["gate"], sh["inner"]), (sh["up"], sh["inner"])))
+            self.shared_down = Linear(sh["inner"], width, sh["down"], None)
 
     def _stacked(self, which):
         E = self.n_experts
@@ -101,11 +149,15 @@ class RoutedExperts(Part):
         specs = self.router.param_specs() + [self._stacked(w) for w in ("gate", "up", "down")]
         if self.correction_name:
             specs.append(ParamSpec(self.correction_name, (self.n_experts,), "vector", ("normal", 0.0, 0.02)))
+        if self.shared:
+            specs += self.shared_up.param_specs() + self.shared_down.param_specs()
         return specs
 
     def bind(self, tensors, runtime):
         super().bind(tensors, runtime)
         self.router.bind(tensors)
+        if self.shared:
+            self.shared_up.bind(tensors), self.shared_down.bind(tensors)
         E = self.n_experts
         self.w_gate = tensors[self.templates["gate"].format(e="*")].view(E, self.inner, self.width)
         self.w_up = tensors[self.templates["up"].format(e="*")].view(E, self.inner, self.width)
@@ -129,15 +181,33 @@ class RoutedExperts(Part):
         wdt = self.w_dtype
         if h.dtype != wdt:        # (experts stored in 32-bit in a bfloat16 engine: their products run on widened rows)
             h = ops.cast(h.contiguous(), torch.empty(h.shape, dtype=wdt, device=dev))
+        returns = accumulate_into is None
+        if returns:
+            accumulate_into = torch.zeros((T, self.width), dtype=torch.float32, device=dev)
         z = self.router(h, out_dtype=torch.float32)
         ids = torch.empty((T, top), dtype=torch.int32, device=dev)
         wts = torch.empty((T, top), dtype=torch.float32, device=dev)
-        ops.moe_route(z, self.correction, top, ids, wts)
+        ops.moe_route(z, self.correction, top, ids, wts, score=self.score, renorm=self.renorm, n_experts=self.n_experts)
         offsets = torch.empty(self.n_experts + 1, dtype=torch.int32, device=dev)
         order = torch.empty(T * top, dtype=torch.int32, device=dev)
         ops.moe_plan(ids, self.n_experts, offsets, order)
         y = torch.empty((T * top, self.inner), dtype=wdt, device=dev)
-        ops.moe_up(h, order, offsets, top, self.w_gate, self.w_up, self.limit, self.alpha, y, dims=self.up_dims)
+        on_input = self.weigh == "input"
+        ops.moe_up(h, order, offsets, top, self.w_gate, self.w_up, self.limit, self.alpha, y, dims=self.up_dims,
+                   kind=self.act, in_scale=wts if on_input else None)
         out = torch.empty((T * top, self.width), dtype=torch.float32, device=dev)
         ops.moe_down(y, order, offsets, self.w_down, out, dims=self.down_dims)
-        ops.moe_combine(out, wts, accumulate_into)
+        ops.moe_combine(out, None if on_input else wts, accumulate_into)
+        if self.shared:
+            n = self.shared["inner"]
+            gu = self.shared_up(h, out_dtype=torch.float32)
+            f = ops.gated(gu[:, n:], gu[:, :n], "silu", torch.empty((T, n), dtype=self.shared_down.weight.dtype, device=dev))
+            s = self.shared_down(f, out_dtype=torch.float32)
+            if self.token_gate:
+                E = self.n_experts
+                share = ops.activate(z[:, E:E + 1], "sigmoid", torch.empty((T, 1), dtype=torch.float32, device=dev))
+                ops.moe_combine(s, share, accumulate_into)
+            else:
+                ops.moe_combine(s, None, accumulate_into)
+        if returns:
+            return accumulate_into

@@ -21,14 +21,26 @@ class CausalSelfAttention(Part):
     position: a position encoding of this layer's own, as (kind name, arguments), of the kind that
     turns queries and keys; None: the model's.
     qkv_weight_sources, qkv_bias_sources: ((file name, columns), ...) where the checkpoint stores the three
-    projections as tensors of their own; qkv_weight / qkv_bias then only name the joined tensors."""
+    projections as tensors of their own; qkv_weight / qkv_bias then only name the joined tensors.
+    value_dim: the width of a value where it is not the keys' (None: head_dim); the output projection then reads
+    n_heads * value_dim columns.  exact_turn: the projection's result stays 32-bit until queries and keys are turned by
+    their positions, so they are rounded once; it is also the way values of another width go (keys and values are then
+    kept side by side in one width, the next multiple of 16 from the wider of the two, the narrower padded with zeros,
+    which add nothing to a score or a result)."""
     graph_safe = True
+    returns_rows = True
 
     def __init__(self, width: int, n_heads: int, n_kv_heads: int, head_dim: int, scale: float,
                  qkv_weight: str, qkv_bias, out_weight: str, out_bias, stored_in_out: bool = False,
                  window: int = 0, out_init_std: float = 0.02, position=None, qkv_weight_sources=None,
-                 qkv_bias_sources=None):
+                 qkv_bias_sources=None, value_dim=None, exact_turn: bool = False):
         self.width, self.n_heads, self.n_kv_heads, self.head_dim = width, n_heads, n_kv_heads, head_dim
+        self.value_dim = head_dim if value_dim is None else int(value_dim)
+        self.split = bool(exact_turn) or self.value_dim != head_dim
+        # (the split way keeps keys and values in one width that every attention kernel takes)
+        self.kept_dim = -(-max(head_dim, self.value_dim) // 16) * 16 if self.split else head_dim
+        if not 1 <= self.kept_dim <= 256:
+            raise ValueError(f"keys of {head_dim} and values of {self.value_dim}: the attention kernels take up to 256")
         self.scale, self.window = float(scale), int(window)
         if n_heads % n_kv_heads != 0:
             raise ValueError(f"{n_heads} heads cannot share {n_kv_heads} key heads")
@@ -36,10 +48,11 @@ class CausalSelfAttention(Part):
             raise ValueError(f"head size {head_dim}: the attention kernels take head sizes up to 256")
         self.q_width = n_heads * head_dim
         self.kv_width = n_kv_heads * head_dim
+        self.v_width = n_kv_heads * self.value_dim
         # (a checkpoint that stores q, k and v apart names them in qkv_*_sources: joined at load, one product here)
-        self.qkv = Linear(width, self.q_width + 2 * self.kv_width, qkv_weight, qkv_bias, stored_in_out,
+        self.qkv = Linear(width, self.q_width + self.kv_width + self.v_width, qkv_weight, qkv_bias, stored_in_out,
                           weight_sources=qkv_weight_sources, bias_sources=qkv_bias_sources)
-        self.out = Linear(self.q_width, width, out_weight, out_bias, stored_in_out, out_init_std)
+        self.out = Linear(n_heads * self.value_dim, width, out_weight, out_bias, stored_in_out, out_init_std)
         self.position = POSITIONS.make(position) if position is not None else None
         if self.position is not None:
             self.graph_safe = getattr(self.position, "graph_safe", False)
@@ -49,7 +62,7 @@ class CausalSelfAttention(Part):
         return self.qkv.param_specs() + self.out.param_specs() + own
 
     def cache_spec(self):
-        return PagedKV(self.n_kv_heads, self.head_dim, self.window)
+        return PagedKV(self.n_kv_heads, self.kept_dim, self.window)
 
     def bind(self, tensors, runtime):
         super().bind(tensors, runtime)
@@ -57,6 +70,7 @@ class CausalSelfAttention(Part):
         self.out.bind(tensors)
         if self.position is not None:
             self.position.bind(tensors, runtime)
+        self.no_freq = torch.empty(0, dtype=torch.float32, device=runtime.device)
 
     def packed_input(self, n_rows):
         return self.qkv.packed_input(n_rows)
@@ -73,10 +87,46 @@ class CausalSelfAttention(Part):
     def defers_sum(self, n_rows):
         return self.out.defers(n_rows)
 
+    def _forward_split(self, h, ctx, cache, g, position, accumulate_into):
+        """The projection's result in 32-bit; queries and keys turned (or copied) from there into rows of the kept width,
+        values copied beside the keys; the cache write, the attention, and the heads' first value_dim columns on."""
+        act, T, dev = self.runtime.act_dtype, h.shape[0], h.device
+        H, G, dk, dv, hw = self.n_heads, self.n_kv_heads, self.head_dim, self.value_dim, self.kept_dim
+        z = self.qkv(h, out_dtype=torch.float32)
+        turns = position is not None and getattr(position, "rotates", False)
+        padded = hw != dk or hw != dv
+        new = torch.zeros if padded else torch.empty
+        q = new((T, H * hw), dtype=act, device=dev)
+        kv = new((T, 2 * G * hw), dtype=act, device=dev)      # keys at column 0, values at G * hw
+
+        def move(n_vec, width, src_off, dst, dst_off, turn):
+            if turn:
+                position.turn(z, dst, ctx.positions, n_vec, width, src_off=src_off, src_stride=width, dst_off=dst_off, dst_stride=hw)
+            else:
+                ops.rotary(z, dst, ctx.positions, self.no_freq, n_vec, 0, width, src_off=src_off, src_stride=width, dst_off=dst_off,
+                           dst_stride=hw)
+        move(H, dk, 0, q, 0, turns)
+        move(G, dk, self.q_width, kv, 0, turns)
+        move(G, dv, self.q_width + self.kv_width, kv, G * hw, False)
+        if cache.writes:
+            ops.kv_write(kv, 0, G * hw, g.slot_map, cache.k, cache.v)
+        o = torch.empty((T, H * hw), dtype=act, device=dev)
+        ops.attention(q, o, cache.k, cache.v, g.block_tables, g.tiles, H, self.scale, self.window, tiles_wide=g.tiles_wide,
+                      single_rows=g.single_rows, max_context=g.max_context)
+        if hw != dv:
+            narrow = torch.empty((T, H * dv), dtype=act, device=dev)
+            ops.rotary(o, narrow, ctx.positions, self.no_freq, H, 0, dv, src_off=0, src_stride=hw, dst_off=0, dst_stride=dv)
+            o = narrow
+        if accumulate_into is None:
+            return self.out(o, out_dtype=torch.float32)
+        self.out(o, residual=accumulate_into)
+
     def forward(self, h, ctx, cache, accumulate_into, stats=None, deferred=None):
         act = self.runtime.act_dtype
         g = ctx.groups[cache.group]
         position = self.position if self.position is not None else self.runtime.position
+        if self.split:
+            return self._forward_split(h, ctx, cache, g, position, accumulate_into)
         if position is not None and getattr(position, "rotates", False):
             # queries and keys are turned by their positions before the keys go to the cache: the
             # product, the turn and the cache write are three steps here, not one kernel
@@ -98,6 +148,8 @@ class CausalSelfAttention(Part):
         ops.attention(q, o, cache.k, cache.v, g.block_tables, g.tiles, self.n_heads,
                       self.scale, self.window, tiles_wide=g.tiles_wide, single_rows=g.single_rows,
                       max_context=g.max_context)
+        if accumulate_into is None:
+            return self.out(o, out_dtype=torch.float32)
         self.out(o, residual=accumulate_into, stats=stats, deferred=deferred)
 
 

@@ -37,6 +37,9 @@ class LayerCall:
     cache: Union[int, Tuple[int, ...]]   # the cache this call uses; a tuple: one for each mixer of the layer
     writes_cache: bool = True     # False: it only reads what another call wrote
     inject: Optional[str] = None  # a name in DecoderSpec.injections: done to the stream right before this call
+    # the checkpoint name of a vector of i + 2 weights for call i of the run order: what goes on behind this call is the sum
+    # of weight[j] * X_j, with X_0 the embedding stage's output and X_(j+1) the stream as call j left it (before its own average)
+    average: Optional[str] = None
 
     def caches(self) -> Tuple[int, ...]:
         return (self.cache,) if isinstance(self.cache, int) else tuple(self.cache)
@@ -181,6 +184,9 @@ class DecoderModel:
             specs.append(ParamSpec(t.name, (t.rows, self.spec.width), "table", ("normal", 0.0, 0.02)))
         for lin in self.injections.values():
             specs += lin.param_specs()
+        for i, call in enumerate(self.spec.run_order):
+            if call.average is not None:
+                specs.append(ParamSpec(call.average, (i + 2,), "vector", ("normal", 1.0 / (i + 2), 0.1)))
         specs += [s for s in self.head.param_specs() if s.name not in seen]     # (a tied head's weight is the table's)
         return specs
 
@@ -194,6 +200,8 @@ class DecoderModel:
         for lin in self.injections.values():
             lin.bind(tensors)
         self.extra_tables = {t.name: tensors[t.name] for t in self.spec.extra_embeddings}
+        self.averages = {i: tensors[c.average] for i, c in enumerate(self.spec.run_order) if c.average is not None}
+        self._one = torch.ones(1, dtype=torch.float32, device=runtime.device) if self.averages else None
         for b in self.blocks:
             after = getattr(b, "after_bind", None)     # an arrangement may make its parts ready for each other
             if after is not None:
@@ -224,7 +232,15 @@ class DecoderModel:
         """ctx: engine.batch.StepContext; cache: cache.storage.CacheStorage.
         -> 32-bit logits [R, vocab] at ctx.logit_rows."""
         rt = self.runtime
-        x = torch.empty((ctx.T, self.spec.width), dtype=torch.float32, device=rt.device)
+        order = self.spec.run_order
+        kept = None
+        if self.averages:
+            # every call's result is kept, plane j + 1 for call j behind the embedding stage's in plane 0; a call works in
+            # its own plane, which holds what went on from the call before
+            kept = torch.empty((len(order) + 2, ctx.T, self.spec.width), dtype=torch.float32, device=rt.device)
+            x = kept[0]
+        else:
+            x = torch.empty((ctx.T, self.spec.width), dtype=torch.float32, device=rt.device)
         if not self.spec.extra_embeddings:
             ops.embed(ctx.tokens, ctx.positions, self.embedding.weight, self.position.table(), x,
                       token_scale=self.spec.embedding_scale)
@@ -238,7 +254,10 @@ class DecoderModel:
         if self.embedding_norm is not None:
             x = self.embedding_norm.forward(x, torch.float32)
         x0 = x.clone() if self.injections else None      # (the blocks add into x in place)
-        order = self.spec.run_order
+        if kept is not None:
+            if x.data_ptr() != kept[0].data_ptr():
+                kept[0].copy_(x)
+            x = ops.depth_mix(kept, 1, self._one, kept[1])
         for i, call in enumerate(order):
             if call.inject is not None:
                 if rt.stream_deferred is not None:
@@ -254,6 +273,14 @@ class DecoderModel:
                 rt.stream_deferred.flush(x)         # (an arrangement that knows nothing of sums left for its norm)
                 rt.stream_deferred = None
             block.forward(x, ctx, [cache.view(c, call.writes_cache) for c in call.caches()], rt)
+            if kept is not None:
+                if rt.stream_deferred is not None:
+                    rt.stream_deferred.flush(x)
+                rt.stream_stats = rt.stream_deferred = None
+                if x.data_ptr() != kept[i + 1].data_ptr():      # (an injection made new rows)
+                    kept[i + 1].copy_(x)
+                w = self.averages.get(i)
+                x = ops.depth_mix(kept, i + 2, w, kept[i + 2]) if w is not None else ops.depth_mix(kept[i + 1:], 1, self._one, kept[i + 2])
         if rt.stream_deferred is not None:
             rt.stream_deferred.flush(x)
         rt.stream_stats = rt.next_norm = rt.stream_deferred = None

@@ -71,3 +71,27 @@ class RMSNorm(Part):
         n = x.shape[0] if rows is None else rows.shape[0]
         out = torch.empty((n, self.width), dtype=out_dtype, device=x.device)
         return ops.rmsnorm(x, self.weight, self.eps, out, rows)
+
+
+@NORMS.register("rmsnorm_into_stream")
+class StreamRMSNorm(RMSNorm):
+    """The norm that stands behind a mixer or a feed-forward, on the result's way into the stream:
+    x += mult * (y / sqrt(mean(y^2) + eps) * weight) * scale, with `scale` a vector of the layer's own (a name, or None)
+    and `mult` a constant of the model.  `add_into(y, x)` does it in one kernel; `forward` is the norm alone."""
+
+    def __init__(self, width: int, eps: float, weight_name: str, scale_name=None, mult: float = 1.0):
+        super().__init__(width, eps, weight_name)
+        self.scale_name, self.mult = scale_name, float(mult)
+
+    def param_specs(self):
+        specs = super().param_specs()
+        if self.scale_name:
+            specs.append(ParamSpec(self.scale_name, (self.width,), "vector", ("normal", 1.0, 0.2)))
+        return specs
+
+    def bind(self, tensors, runtime):
+        super().bind(tensors, runtime)
+        self.scale = tensors[self.scale_name] if self.scale_name else None
+
+    def add_into(self, y, x):
+        return ops.rmsnorm_add(y, self.weight, self.scale, self.mult, self.eps, x)

@@ -113,3 +113,140 @@ class HGRN2(Part):
         y = torch.empty((T, self.vw), dtype=act, device=h.device)
         ops.head_norm(o, self.norm, self.eps, y, self.n_heads)
         self.out(y, residual=accumulate_into)
+
+
+@MIXERS.register("lightning")
+class Lightning(Part):
+    """A matrix per head that fades by a constant of the head: q, k and v go through silu, S <- decay_h S + k v^T, o = S^T q
+    (the token's own write is read).  All heads' o are normed together as one vector with a weight per column, times
+    sigmoid(W_g h), then the output projection.  State: S in 32-bit."""
+    graph_safe = True
+    returns_rows = True
+    libraries = ("sequence",)
+
+    def __init__(self, width: int, n_heads: int, head_dim: int, value_dim: int, decay, eps: float, names: dict):
+        """decay: a number per head; names: q, k, v, g, o (matrices); norm (vector)."""
+        self.width, self.n_heads, self.head_dim, self.value_dim, self.eps = width, n_heads, head_dim, value_dim, eps
+        self.decay = [float(d) for d in decay]
+        if len(self.decay) != n_heads:
+            raise ValueError(f"lightning: {len(self.decay)} decays for {n_heads} heads")
+        self.names = dict(names)
+        self.qk, self.vw = n_heads * head_dim, n_heads * value_dim
+        self.proj = Linear(width, 2 * self.qk + 2 * self.vw, names["q"] + "+k+v+g", None,
+                           weight_sources=((names["q"], self.qk), (names["k"], self.qk), (names["v"], self.vw), (names["g"], self.vw)))
+        self.out = Linear(self.vw, width, names["o"], None)
+
+    def param_specs(self):
+        return self.proj.param_specs() + self.out.param_specs() + [
+            ParamSpec(self.names["norm"], (self.vw,), "vector", ("normal", 1.0, 0.1))]
+
+    def cache_spec(self):
+        return FixedState((self.qk * self.value_dim,))
+
+    def bind(self, tensors, runtime):
+        super().bind(tensors, runtime)
+        self.proj.bind(tensors), self.out.bind(tensors)
+        self.norm = tensors[self.names["norm"]]
+        self.decay_t = torch.tensor(self.decay, dtype=torch.float64).to(F32).to(runtime.device)
+
+    def forward(self, h, ctx, cache, accumulate_into):
+        act, T, qk, vw = self.runtime.act_dtype, h.shape[0], self.qk, self.vw
+        z = self.proj(h, out_dtype=F32)
+        qkv = z[:, :2 * qk + vw]
+        ops.activate(qkv, "silu", qkv)
+        o = torch.empty((T, vw), dtype=F32, device=h.device)
+        ops.state_scan(z[:, :qk], z[:, qk:2 * qk], z[:, 2 * qk:2 * qk + vw], None, None, cache.state, ctx.row_start, ctx.state_slots,
+                       self.n_heads, self.head_dim, self.value_dim, o, read_after=True, w_head=self.decay_t)
+        y = torch.empty((T, vw), dtype=act, device=h.device)
+        ops.head_norm(o, self.norm, self.eps, y, 1, gate=z[:, 2 * qk + vw:], gate_kind="sigmoid")
+        if accumulate_into is None:
+            return self.out(y, out_dtype=F32)
+        self.out(y, residual=accumulate_into)
+
+
+@MIXERS.register("channel_delta")
+class ChannelDelta(Part):
+    """The delta rule with a decay per head and key channel.  q and k (n_qk_heads heads of head_dim) and v (n_heads of
+    value_dim) each pass a short causal convolution over time on every channel and silu; q and k are made unit vectors per
+    head (x / sqrt(sum x^2 + 1e-6)), q times head_dim^(-1/2); head h reads q and k of head h // (n_heads // n_qk_heads).
+    beta = sigmoid(W_b h) per head; the decay g = exp(-exp(A_log_h) * softplus(W_a2 W_a1 h + dt_bias)) per head and key
+    channel.  Per head: S <- diag(g) S; e = beta (v - S^T k); S <- S + k e^T; o = S^T q.  Each head's o is divided by its
+    root mean square, times a weight per value column that the heads share, times sigmoid(W_g2 W_g1 h); then the output
+    projection.  State: S in 32-bit and the convolutions' last taps - 1 inputs."""
+    graph_safe = True
+    returns_rows = True
+    libraries = ("sequence",)
+    UNIT_EPS = 1e-6
+
+    def __init__(self, width: int, n_heads: int, n_qk_heads: int, head_dim: int, value_dim: int, taps: int, eps: float,
+                 decay_rank: int, gate_rank: int, names: dict):
+        """names: q, k, v, b, a1, a2, g1, g2, o (matrices); q_conv, k_conv, v_conv ([channels, taps]); A_log, dt_bias, norm."""
+        if n_heads % n_qk_heads != 0:
+            raise ValueError(f"channel_delta: {n_heads} heads cannot share {n_qk_heads} heads of queries and keys")
+        if taps < 1:
+            raise ValueError(f"channel_delta: {taps} taps")
+        self.width, self.n_heads, self.n_qk_heads, self.head_dim, self.value_dim = width, n_heads, n_qk_heads, head_dim, value_dim
+        self.taps, self.eps, self.names = taps, eps, dict(names)
+        self.qk, self.vw, self.gw = n_qk_heads * head_dim, n_heads * value_dim, n_heads * head_dim
+        self.channels = 2 * self.qk + self.vw
+        self.decay_rank, self.gate_rank = decay_rank, gate_rank
+        n = names
+        # one product for everything that reads h: q | k | v | b | a1 | g1
+        self.proj = Linear(width, self.channels + n_heads + decay_rank + gate_rank, n["q"] + "+k+v+b+a1+g1", None,
+                           weight_sources=((n["q"], self.qk), (n["k"], self.qk), (n["v"], self.vw), (n["b"], n_heads),
+                                           (n["a1"], decay_rank), (n["g1"], gate_rank)))
+        self.a2 = Linear(decay_rank, self.gw, n["a2"], None)
+        self.g2 = Linear(gate_rank, self.vw, n["g2"], None)
+        self.out = Linear(self.vw, width, n["o"], None)
+
+    def param_specs(self):
+        n, taps = self.names, self.taps
+        specs = []
+        for lin in (self.proj, self.a2, self.g2, self.out):
+            specs += lin.param_specs()
+        return specs + [
+            ParamSpec(n["q_conv"] + "+k+v", (self.channels, taps), "vector", ("normal", 0.0, 0.4),
+                      sources=((n["q_conv"], self.qk), (n["k_conv"], self.qk), (n["v_conv"], self.vw))),
+            ParamSpec(n["A_log"], (self.n_heads,), "vector", ("uniform", -2.0, 0.5)),
+            ParamSpec(n["dt_bias"], (self.gw,), "vector", ("normal", -1.0, 1.0)),
+            ParamSpec(n["norm"], (self.value_dim,), "vector", ("normal", 1.0, 0.1))]
+
+    def cache_spec(self):
+        return FixedState((self.gw * self.value_dim + (self.taps - 1) * self.channels,))
+
+    def bind(self, tensors, runtime):
+        super().bind(tensors, runtime)
+        for lin in (self.proj, self.a2, self.g2, self.out):
+            lin.bind(tensors)
+        n = self.names
+        self.conv = tensors[n["q_conv"] + "+k+v"]
+        self.dt_bias, self.norm = tensors[n["dt_bias"]], tensors[n["norm"]]
+        # the decay's rate per head, spread over the head's key channels
+        self.rate = torch.exp(tensors[n["A_log"]].to(F32)).repeat_interleave(self.head_dim).contiguous()
+
+    def forward(self, h, ctx, cache, accumulate_into):
+        act, T, dev = self.runtime.act_dtype, h.shape[0], h.device
+        qk, vw, C, H = self.qk, self.vw, self.channels, self.n_heads
+        n_state = self.gw * self.value_dim
+        state, past = cache.state[:, :n_state], cache.state[:, n_state:]
+        z = self.proj(h, out_dtype=F32)
+        x = torch.empty((T, C), dtype=F32, device=dev)
+        ops.conv_rows(z[:, :C], self.conv, past, ctx.row_start, ctx.state_slots, x, identity=False, act="silu")
+        if self.taps > 1 and cache.writes:
+            ops.history_update(z[:, :C], past, ctx.row_start, ctx.state_slots)
+        q, k, v = x[:, :qk], x[:, qk:2 * qk], x[:, 2 * qk:]
+        ops.unit_heads(q, self.n_qk_heads, self.head_dim, self.UNIT_EPS, self.head_dim ** -0.5, q)
+        ops.unit_heads(k, self.n_qk_heads, self.head_dim, self.UNIT_EPS, 1.0, k)
+        beta = ops.activate(z[:, C:C + H], "sigmoid", torch.empty((T, H), dtype=F32, device=dev))
+        low = C + H
+        g = self.a2(z[:, low:low + self.decay_rank].contiguous(), out_dtype=F32)
+        ops.activate(g, "exp_neg_softplus", g, bias=self.dt_bias, lower=self.rate)
+        gate = self.g2(z[:, low + self.decay_rank:].contiguous(), out_dtype=F32)
+        o = torch.empty((T, vw), dtype=F32, device=dev)
+        ops.state_scan(q, k, v, g, None, state, ctx.row_start, ctx.state_slots, H, self.head_dim, self.value_dim, o, beta=beta,
+                       qk_heads=self.n_qk_heads)
+        y = torch.empty((T, vw), dtype=act, device=dev)
+        ops.head_norm(o, self.norm, self.eps, y, H, gate=gate, gate_kind="sigmoid")
+        if accumulate_into is None:
+            return self.out(y, out_dtype=F32)
+        self.out(y, residual=accumulate_into)

@@ -236,6 +236,11 @@ def _act(kind, z, lower=None):
         return torch.exp(-torch.exp(z))
     if kind == "bounded_sigmoid":
         return lower + (1.0 - lower) * torch.sigmoid(z)
+    if kind == "exp_neg_softplus":
+        return torch.exp(-lower * torch.nn.functional.softplus(z))
+    if kind == "xielu":
+        neg = torch.clamp(z, max=0)
+        return torch.where(z > 0, lower[0] * z * z + 0.5 * z, lower[1] * (torch.expm1(neg) - neg) + 0.5 * z)
     raise ValueError(kind)
 
 
@@ -244,6 +249,33 @@ def rmsnorm(x, weight, eps, out, rows=None):
     src = (x if rows is None else x[rows.long()])[:, :E].float()
     y = src / torch.sqrt((src * src).mean(dim=-1, keepdim=True) + eps)
     out.copy_(y if weight is None else y * weight)
+    return out
+
+
+def rmsnorm_add(y, weight, scale, mult, eps, x):
+    src = y.float()
+    n = src / torch.sqrt((src * src).mean(dim=-1, keepdim=True) + eps)
+    if weight is not None:
+        n = n * weight
+    if scale is not None:
+        n = n * scale
+    x += mult * n
+    return x
+
+
+def depth_mix(hist, n, weights, out):
+    acc = torch.zeros_like(hist[0])
+    for j in range(n):
+        acc = acc + weights[j] * hist[j]
+    out.copy_(acc)
+    return out
+
+
+def unit_heads(x, n_heads, dim, eps, scale, out):
+    T = x.shape[0]
+    v = x[:, :n_heads * dim].reshape(T, n_heads, dim)
+    y = v / torch.sqrt((v * v).sum(dim=-1, keepdim=True) + eps) * scale
+    out[:, :n_heads * dim] = y.reshape(T, n_heads * dim)
     return out
 
 
@@ -257,17 +289,18 @@ def _requests(row_start, slots):
     return [(sl[s], rs[s], rs[s + 1]) for s in range(len(sl)) if sl[s] >= 0]
 
 
-def conv_rows(h, w, hist, row_start, slots, out):
+def conv_rows(h, w, hist, row_start, slots, out, identity=True, act=None):
     width, taps = w.shape
-    res = torch.zeros(h.shape, dtype=torch.float32)
+    h = h[:, :width]
+    res = torch.zeros((h.shape[0], width), dtype=torch.float32)
     for slot, a, b in _requests(row_start, slots):
         rows = h[a:b] if taps == 1 else torch.cat([hist[slot].view(taps - 1, width), h[a:b]], dim=0)
         for t in range(b - a):
-            acc = h[a + t].clone()
+            acc = h[a + t].clone() if identity else torch.zeros(width)
             for j in range(taps):
                 acc += w[:, j] * rows[t + j]
             res[a + t] = acc
-    out.copy_(res)
+    out.copy_(res if act is None else _act(act, res))
     return out
 
 
@@ -315,15 +348,24 @@ def gated(x, g, kind, out):
     return out
 
 
-def state_scan(r, k, v, w, u, state, row_start, slots, n_heads, dk, dv, out, read_after=False, key_from_decay=False):
+def state_scan(r, k, v, w, u, state, row_start, slots, n_heads, dk, dv, out, read_after=False, key_from_decay=False, beta=None,
+               w_head=None, qk_heads=None):
     H = n_heads
+    G = H if qk_heads is None else qk_heads
+    spread = lambda x: x.view(G, dk).repeat_interleave(H // G, dim=0)      # noqa: E731  (head h reads head h // (H // G))
     for slot, a, b in _requests(row_start, slots):
         S = state[slot].view(H, dv, dk).transpose(1, 2).clone()      # (held [head][value column][key channel])
         for t in range(a, b):
-            rt, wt, vt = r[t].view(H, dk), w[t].view(H, dk), v[t].view(H, dv)
-            at = (1.0 - wt) if key_from_decay else k[t].view(H, dk)
+            rt, vt = spread(r[t]), v[t].view(H, dv)
+            wt = w[t].view(H, dk) if w is not None else w_head.view(H, 1).expand(H, dk)
+            at = (1.0 - wt) if key_from_decay else spread(k[t])
             kv = at[:, :, None] * vt[:, None, :]
-            if read_after:
+            if beta is not None:
+                S = wt[:, :, None] * S
+                e = beta[t].view(H, 1) * (vt - torch.einsum("hi,hij->hj", at, S))
+                S = S + at[:, :, None] * e[:, None, :]
+                out[t] = torch.einsum("hi,hij->hj", rt, S).reshape(-1)
+            elif read_after:
                 S = wt[:, :, None] * S + kv
                 out[t] = torch.einsum("hi,hij->hj", rt, S).reshape(-1)
             else:
@@ -358,8 +400,10 @@ def heads_linear(a, w, out, a_off=0, a_stride=None, o_off=0, o_stride=None):
     return out
 
 
-def moe_route(z, correction, top, ids, wts):
-    s = torch.softmax(z, dim=-1)
+def moe_route(z, correction, top, ids, wts, score="softmax", renorm=True, n_experts=None):
+    if n_experts is not None:
+        z = z[:, :n_experts]
+    s = torch.softmax(z, dim=-1) if score == "softmax" else torch.sigmoid(z)
     choice = s if correction is None else s + correction
     for t in range(z.shape[0]):
         c = choice[t].clone()
@@ -370,7 +414,7 @@ def moe_route(z, correction, top, ids, wts):
             c[e] = -float("inf")
         ws = s[t, picked]
         ids[t] = torch.tensor(picked, dtype=torch.int32)
-        wts[t] = ws / (ws.sum() + 1e-20)
+        wts[t] = ws / (ws.sum() + 1e-20) if renorm else ws
 
 
 def moe_plan(ids, n_experts, offsets, order):
@@ -382,12 +426,17 @@ def moe_plan(ids, n_experts, offsets, order):
     offsets[1:] = torch.cumsum(counts, 0).to(torch.int32)
 
 
-def moe_up(h, order, offsets, top, w_gate, w_up, limit, alpha, y, dims=None):
+def moe_up(h, order, offsets, top, w_gate, w_up, limit, alpha, y, dims=None, kind="clamped", in_scale=None):
     assert dims is None, "packed experts are for the GPU's kernels"
     off = offsets.tolist()
     for e in range(w_gate.shape[0]):
         for p in range(off[e], off[e + 1]):
             x = h[int(order[p]) // top].float()
+            if kind == "silu":
+                sc = 1.0 if in_scale is None else in_scale.reshape(-1)[int(order[p])]
+                g, u = (w_gate[e].float() @ x) * sc, (w_up[e].float() @ x) * sc
+                y[p] = (g * torch.sigmoid(g) * u).to(y.dtype)
+                continue
             g = torch.clamp(w_gate[e].float() @ x, max=limit)
             u = torch.clamp(w_up[e].float() @ x, min=-limit, max=limit)
             y[p] = (g * torch.sigmoid(alpha * g) * (u + 1.0)).to(y.dtype)
@@ -402,5 +451,9 @@ def moe_down(y, order, offsets, w_down, out, dims=None):
 
 
 def moe_combine(out, wts, x):
-    T, top = wts.shape
+    T = x.shape[0]
+    if wts is None:
+        x += out.view(T, -1, x.shape[1]).sum(dim=1)
+        return
+    top = wts.shape[1]
     x += (out.view(T, top, -1) * wts[:, :, None]).sum(dim=1)
