@@ -129,12 +129,13 @@ class RoutedExperts(Part):
         self.token_gate = self.shared.get("token_gate") if self.shared else None
         # the router, and behind its rows the shared expert's gate: one product for both
         if self.token_gate:
-            self.router = Linear(width, n_experts + 1, router + "+gate", None, weight_sources=((router, n_experts), (self.token_gate, 1)))
+            self.router = Linear(width, n_experts + 1, router + "+gate", None, init_std=width ** -0.5,
+                                 weight_sources=((router, n_experts), (self.token_gate, 1)))
         else:
             self.router = Linear(width, n_experts, router, None)
         if self.shared:
             sh = self.shared
-            self.shared_up = Linear(width, 2 * sh["inner"], sh["gate"] + "+up", None,
+            self.shared_up = Linear(width, 2 * sh["inner"], sh["gate"] + "+up", None, init_std=width ** -0.5,
                                     weight_sources=((sh["gate"], sh["inner"]), (sh["up"], sh["inner"])))
             self.shared_down = Linear(sh["inner"], width, sh["down"], None)
 

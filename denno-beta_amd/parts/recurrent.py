@@ -132,7 +132,7 @@ class Lightning(Part):
             raise ValueError(f"lightning: {len(self.decay)} decays for {n_heads} heads")
         self.names = dict(names)
         self.qk, self.vw = n_heads * head_dim, n_heads * value_dim
-        self.proj = Linear(width, 2 * self.qk + 2 * self.vw, names["q"] + "+k+v+g", None,
+        self.proj = Linear(width, 2 * self.qk + 2 * self.vw, names["q"] + "+k+v+g", None, init_std=width ** -0.5,
                            weight_sources=((names["q"], self.qk), (names["k"], self.qk), (names["v"], self.vw), (names["g"], self.vw)))
         self.out = Linear(self.vw, width, names["o"], None)
 
@@ -193,10 +193,10 @@ class ChannelDelta(Part):
         n = names
         # one product for everything that reads h: q | k | v | b | a1 | g1
         self.proj = Linear(width, self.channels + n_heads + decay_rank + gate_rank, n["q"] + "+k+v+b+a1+g1", None,
-                           weight_sources=((n["q"], self.qk), (n["k"], self.qk), (n["v"], self.vw), (n["b"], n_heads),
+                           init_std=width ** -0.5, weight_sources=((n["q"], self.qk), (n["k"], self.qk), (n["v"], self.vw), (n["b"], n_heads),
                                            (n["a1"], decay_rank), (n["g1"], gate_rank)))
-        self.a2 = Linear(decay_rank, self.gw, n["a2"], None)
-        self.g2 = Linear(gate_rank, self.vw, n["g2"], None)
+        self.a2 = Linear(decay_rank, self.gw, n["a2"], None, init_std=decay_rank ** -0.5)
+        self.g2 = Linear(gate_rank, self.vw, n["g2"], None, init_std=gate_rank ** -0.5)
         self.out = Linear(self.vw, width, n["o"], None)
 
     def param_specs(self):

@@ -89,7 +89,14 @@ def test_rotary(dtype, dims, width):
 def test_activate_and_gated(kind):
     x = torch.randn(6, 45, device=DEV) * 2
     bias, lower = torch.randn(45, device=DEV), torch.rand(45, device=DEV)
+    if kind == "xielu":      # (two numbers for all columns)
+        lower = (lower[:2] + 0.3).contiguous()
     both("activate", lambda: (x, kind, torch.empty(6, 45, device=DEV), bias, lower), [2])
+    # the columns of wider rows, in place
+    wide = torch.randn(6, 60, device=DEV)
+    want = ref.activate(wide[:, 5:50].cpu(), kind, torch.empty(6, 45), bias.cpu(), lower.cpu())
+    ops.activate(wide[:, 5:50], kind, wide[:, 5:50], bias, lower)
+    close(wide[:, 5:50], want)
     if kind in ("silu", "sigmoid", "tanh"):
         g = torch.randn(6, 45, device=DEV)
         both("gated", lambda: (x.bfloat16(), g, kind, torch.empty(6, 45, dtype=torch.bfloat16, device=DEV)), [3], torch.bfloat16)
@@ -115,6 +122,132 @@ def test_state_scan(dk, dv, heads, mode, lengths):
             return (r, k, v, w, u, st[:, :heads * dk * dv], row_start, slots, heads, dk, dv, out, False, False)
         return (r, None, v, w, None, st[:, :heads * dk * dv], row_start, slots, heads, dk, dv, out, True, True)
     both("state_scan", make, [5, 11])
+
+
+@pytest.mark.parametrize("dk,dv,heads,qk_heads", [(16, 16, 2, 2), (48, 32, 4, 2), (5, 70, 1, 1), (64, 64, 4, 1), (100, 9, 2, 2), (130, 20, 3, 1),
+                                                  (32, 12, 6, 3), (128, 36, 1, 1), (252, 8, 1, 1), (64, 128, 2, 2), (6, 10, 2, 1)])
+@pytest.mark.parametrize("lengths", [[1, 12, 40], [1, 2, 1]])
+def test_state_scan_delta_rule(dk, dv, heads, qk_heads, lengths):
+    """S <- diag(w) S; e = beta (v - S^T k); S <- S + k e^T; o = S^T r, with fewer heads of r and k than of v."""
+    row_start, slots, T = tables(lengths, [2, -1, 0])
+    wide = torch.randn(T, 4 + 2 * qk_heads * dk, device=DEV)                  # r and k: columns of wider rows
+    r, k = wide[:, :qk_heads * dk], wide[:, qk_heads * dk:2 * qk_heads * dk]
+    k = torch.nn.functional.normalize(k.reshape(T, qk_heads, dk), dim=-1).reshape(T, -1).contiguous()
+    v = torch.randn(T, heads * dv, device=DEV)
+    w = torch.rand(T, heads * dk, device=DEV) * 0.5 + 0.5
+    beta = torch.rand(T, heads, device=DEV)
+    state = torch.randn(3, heads * dk * dv + 11, device=DEV)
+
+    def make():
+        st = state.clone()
+        return (r, k, v, w, None, st[:, :heads * dk * dv], row_start, slots, heads, dk, dv, torch.zeros(T, heads * dv, device=DEV), False,
+                False, beta, None, qk_heads)
+    both("state_scan", make, [5, 11])
+
+
+@pytest.mark.parametrize("dk,dv,heads", [(16, 8, 2), (40, 24, 1), (64, 64, 3), (7, 5, 2)])
+@pytest.mark.parametrize("lengths", [[3, 1, 50], [1, 1, 1]])
+def test_state_scan_with_one_decay_a_head(dk, dv, heads, lengths):
+    row_start, slots, T = tables(lengths, [1, 0, -1])
+    r, k, v = (torch.randn(T, heads * n, device=DEV) for n in (dk, dk, dv))
+    decay = torch.rand(heads, device=DEV) * 0.6 + 0.4
+    state = torch.randn(2, heads * dk * dv, device=DEV)
+    both("state_scan", lambda: (r, k, v, None, None, state.clone(), row_start, slots, heads, dk, dv, torch.zeros(T, heads * dv, device=DEV),
+                                True, False, None, decay), [5, 11])
+
+
+@pytest.mark.parametrize("taps", [1, 2, 4])
+def test_conv_without_the_row_itself_then_silu(taps):
+    """The channels are the first columns of wider rows; the history is kept from the same columns."""
+    width = 41
+    row_start, slots, T = tables([1, 7, 2, 3], [2, 0, -1, 3])
+    h = torch.randn(T, width + 9, device=DEV)
+    w = torch.randn(width, taps, device=DEV)
+    hist = torch.randn(5, max(taps - 1, 1) * width + 6, device=DEV)[:, 6:6 + (taps - 1) * width]
+    both("conv_rows", lambda: (h[:, :width], w, hist, row_start, slots, torch.zeros(T, width, device=DEV), False, "silu"), [5])
+    both("conv_rows", lambda: (h[:, :width], w, hist, row_start, slots, torch.zeros(T, width, device=DEV), False, None), [5])
+    if taps > 1:
+        mine, theirs = hist.clone(), hist.cpu().clone()
+        ops.history_update(h[:, :width], mine, row_start, slots)
+        ref.history_update(h[:, :width].cpu(), theirs, row_start.cpu(), slots.cpu())
+        close(mine, theirs)
+
+
+@pytest.mark.parametrize("width", [7, 96, 1000])
+@pytest.mark.parametrize("dtype", DT)
+def test_norm_added_into_the_stream(width, dtype):
+    y = (torch.randn(11, width, device=DEV) * 3).to(dtype)
+    w, scale = torch.randn(width, device=DEV), torch.randn(width, device=DEV)
+    x = torch.randn(11, width + 3, device=DEV)
+    both("rmsnorm_add", lambda: (y, w, scale, 0.37, 1e-5, x[:, :width].clone()), [5])
+    both("rmsnorm_add", lambda: (y, None, None, 1.0, 1e-3, x[:, :width].clone()), [5])
+
+
+@pytest.mark.parametrize("T,width", [(5, 32), (3, 7), (40, 100)])
+def test_average_over_depth(T, width):
+    planes = 6
+    hist = torch.randn(planes, T, width, device=DEV)
+    weights = torch.randn(planes, device=DEV)
+    for n in (1, 2, 5):
+        mine, theirs = hist.clone(), hist.cpu().clone()
+        ops.depth_mix(mine, n, weights, mine[n])              # (into the next plane)
+        ref.depth_mix(theirs, n, weights.cpu(), theirs[n])
+        close(mine, theirs)
+    both("depth_mix", lambda: (hist, planes, weights, torch.empty(T, width, device=DEV)), [3])
+
+
+def test_unit_vectors_per_head():
+    T, H, dim = 9, 3, 20
+    x = torch.randn(T, H * dim + 5, device=DEV)
+    both("unit_heads", lambda: (x[:, :H * dim], H, dim, 1e-6, dim ** -0.5, torch.zeros(T, H * dim, device=DEV)), [5])
+    tiny = x * 1e-4                                              # (the eps counts where the vector is short)
+    both("unit_heads", lambda: (tiny[:, :H * dim], H, dim, 1e-6, 1.0, torch.zeros(T, H * dim, device=DEV)), [5])
+    mine = x.clone()
+    ops.unit_heads(mine[:, :H * dim], H, dim, 1e-6, 1.0, mine[:, :H * dim])
+    close(mine[:, :H * dim], ref.unit_heads(x[:, :H * dim].cpu(), H, dim, 1e-6, 1.0, torch.zeros(T, H * dim)))
+    close(mine[:, H * dim:], x[:, H * dim:])
+
+
+@pytest.mark.parametrize("T,E,top", [(1, 4, 2), (50, 16, 3), (33, 70, 1), (9, 5, 5)])
+def test_route_by_sigmoid_scores_as_they_are(T, E, top):
+    z = torch.randn(T, E + 2, device=DEV) * 2                   # (further columns behind the experts')
+    ids, wts = torch.zeros(T, top, dtype=torch.int32, device=DEV), torch.zeros(T, top, device=DEV)
+    ops.moe_route(z, None, top, ids, wts, score="sigmoid", renorm=False, n_experts=E)
+    hi, hw = torch.zeros(T, top, dtype=torch.int32), torch.zeros(T, top)
+    ref.moe_route(z.cpu(), None, top, hi, hw, score="sigmoid", renorm=False, n_experts=E)
+    assert torch.equal(ids.cpu(), hi)
+    close(wts, hw)
+    close(wts, torch.sigmoid(z[:, :E]).cpu().gather(1, hi.long()))
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("T,E,top,ff,width", [(1, 3, 2, 8, 24), (45, 6, 3, 70, 50), (200, 5, 2, 64, 128), (9, 8, 2, 96, 64), (3, 40, 1, 32, 160)])
+def test_experts_that_read_weighted_rows(dtype, T, E, top, ff, width):
+    """silu(W_gate s h) * (W_up s h) with a factor s per (token, choice); weights None in the sum of a token's results."""
+    h = torch.randn(T, width, device=DEV).to(dtype)
+    wg, wu = ((torch.randn(E, ff, width, device=DEV) / width ** 0.5).to(dtype) for _ in range(2))
+    ids = torch.stack([torch.randperm(E, device=DEV)[:top] for _ in range(T)]).int()
+    offsets, order = torch.zeros(E + 1, dtype=torch.int32, device=DEV), torch.zeros(T * top, dtype=torch.int32, device=DEV)
+    ops.moe_plan(ids, E, offsets, order)
+    s = torch.rand(T, top, device=DEV) + 0.2
+    for scale in (s, None):
+        y = torch.zeros(T * top, ff, dtype=dtype, device=DEV)
+        ops.moe_up(h, order, offsets, top, wg, wu, 0.0, 1.0, y, kind="silu", in_scale=scale)
+        hy = torch.zeros(T * top, ff, dtype=dtype)
+        ref.moe_up(h.cpu(), order.cpu(), offsets.cpu(), top, wg.cpu(), wu.cpu(), 0.0, 1.0, hy, kind="silu",
+                   in_scale=None if scale is None else scale.cpu())
+        close(y, hy, dtype, "moe_up")
+        if dtype == torch.bfloat16 and ops.experts_packable(E, ff, width):
+            y2 = torch.zeros_like(y)
+            ops.moe_up(h, order, offsets, top, ops.pack_matrix(wg.view(E * ff, width)), ops.pack_matrix(wu.view(E * ff, width)), 0.0, 1.0,
+                       y2, dims=(E, ff, width), kind="silu", in_scale=scale)
+            close(y2, hy, dtype, "moe_up, packed")
+    out = torch.randn(T * top, width, device=DEV)
+    x = torch.randn(T, width, device=DEV)
+    hx = x.cpu().clone()
+    ops.moe_combine(out, None, x)
+    ref.moe_combine(out.cpu(), None, hx)
+    close(x, hx)
 
 
 @pytest.mark.parametrize("dtype", DT)
