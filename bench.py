@@ -18,6 +18,9 @@ decode steps and prefill (`fp32`).  Peaks are the published ones of MI355X.
     python bench.py --only ridopel [--width 1024] [--kernel-times]   four Ridopel layers (latent attention, hgrn2, latent
                                                              attention, wkv, each with sixteen experts) beside four GPT-2
                                                              layers of the same width: prefill and decode
+    python bench.py --only pafivik [--width 1024] [--kernel-times]   four Pafivik layers (lightning, channel_delta, attention,
+                                                             channel_delta, each with sixteen experts and a shared one) beside
+                                                             four Ridopel layers of the same width: prefill and decode
 """
 import argparse
 import json
@@ -187,8 +190,8 @@ def main():
     ap.add_argument("--shape", choices=["xl", "large", "medium"], default=None,
                     help="--only decode / prefill / replay: the layer sizes of BASELINE.json's configs[2], [3] or [4] "
                          "(default xl; for replay medium)")
-    ap.add_argument("--width", type=int, default=0, help="--only ridopel: one width instead of 1,024 and 2,048")
-    ap.add_argument("--only", choices=["decode", "prefill", "serving", "replay", "ridopel"], default=None,
+    ap.add_argument("--width", type=int, default=0, help="--only ridopel, --only pafivik: one width instead of 1,024 and 2,048")
+    ap.add_argument("--only", choices=["decode", "prefill", "serving", "replay", "ridopel", "pafivik"], default=None,
                     help="run one workload and print a short line (decode, prefill: for profiling; serving: "
                          "BASELINE.json's configs[3], GPT-2 Large shape, 64 requests through the scheduler; replay: "
                          "configs[4], GPT-2 Medium shape, against the plain implementation)")
@@ -200,6 +203,8 @@ def main():
         return serving(a)
     if a.only == "ridopel":
         return ridopel(a)
+    if a.only == "pafivik":
+        return pafivik(a)
     if a.only == "replay":
         a.shape = a.shape or "medium"      # (configs[4] as written; --shape xl: the same replay at configs[2]'s sizes)
         return replay(a)
@@ -277,14 +282,44 @@ def ridopel_configs(width, layers=4, vocab=32000, positions=2048):
     return rid, gpt
 
 
+def pafivik_configs(width, layers=4, vocab=32000, positions=2048):
+    """-> (a Pafivik config, a Ridopel config) of the same width, layers, vocabulary and positions.  The Pafivik layers
+    take turns between lightning (heads of 64 keys x 128 values), channel_delta (as many heads of 64 x 128 over half as many
+    heads of queries and keys, four taps, inner sizes of 64), attention (heads of 64, a key head for every four, all 64
+    dimensions turned) and channel_delta again; each has sixteen experts of the model's width of which a token uses two, and
+    a shared expert of the model's width: Ridopel's experts, so that the two differ by their mixers, norms and averages."""
+    H = width // 128
+    moe = dict(kind="moe", expert=dict(ff=width), router=dict(experts=16, top=2), shared=dict(ff=width))
+    delta = dict(type="channel_delta", mlp=moe, mixer=dict(heads=H, kv_heads=max(1, H // 2), dim=64, vdim=128, conv=4, decay_rank=64,
+                                                             gate_rank=64))
+    kinds = [dict(type="lightning", mlp=moe, mixer=dict(heads=H, dim=64, vdim=128, decay=[1.0 - 2.0 ** -(5 + 3 * h / H) for h in range(H)])),
+             delta,
+             dict(type="attention", mlp=moe, mixer=dict(heads=width // 64, kv_heads=max(1, width // 256), dim=64, vdim=64, scale=0.125,
+                                                        rot=dict(base=10000.0, dims=64))),
+             delta]
+    paf = dict(architecture="Pafivik", vocab=vocab, width=width, norm=dict(eps=1e-5), embedding=dict(scale=1.0), residual_mult=0.5,
+               layers=[kinds[i % 4] for i in range(layers)], max_positions=positions, n_positions=positions, vocab_size=vocab)
+    return paf, ridopel_configs(width, layers, vocab, positions)[0]
+
+
+def pafivik(a):
+    """Prefill and decode steps of four Pafivik layers beside four Ridopel layers of the same width (the closest of the
+    framework's models: recurrent mixers, an attention, the same experts); with --kernel-times each model's kernels."""
+    return side_by_side(a, ("pafivik", "ridopel"), pafivik_configs)
+
+
 def ridopel(a):
     """Prefill (two prompts of 1,024 tokens in one step) and decode steps (batch 8 and 64 from a context of 512) of four
     Ridopel layers beside four GPT-2 layers of the same width; with --kernel-times each model's kernels, launch by launch."""
+    return side_by_side(a, ("ridopel", "gpt2"), ridopel_configs)
+
+
+def side_by_side(a, names, configs):
     import torch
     from denno_beta_amd.kernels import ops
     out = {}
     for width in ([a.width] if a.width else [1024, 2048]):
-        for name, cfg in zip(("ridopel", "gpt2"), ridopel_configs(width, a.layers or 4)):
+        for name, cfg in zip(names, configs(width, a.layers or 4)):
             w = Workloads(a, a.dtype, cfg)
             rec = {"weight_bytes": w.runner.model.weight_bytes(), "cache_bytes_per_token": w.runner.cache.bytes_per_token()}
             w.prefill(1, a.prompts)

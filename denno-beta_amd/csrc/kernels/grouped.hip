@@ -329,11 +329,17 @@ __global__ __launch_bounds__(256) void expert_down_kernel(const void* y, int y_d
 }
 
 // x[t, :] += sum_c wts[t, c] * out[t * top + c, :], the choices in their order (wts none: every weight is 1)
-__global__ __launch_bounds__(256) void combine_kernel(const float* out, const float* wts, int top, int width, float* x, size_t ldx) {
+// (logits: a weight is sigmoid of what wts holds; the weights of a row are then ldw numbers apart)
+__global__ __launch_bounds__(256) void combine_kernel(const float* out, const float* wts, size_t ldw, int logits, int top, int width,
+                                                      float* x, size_t ldx) {
   const int t = blockIdx.x;
   for (int c = threadIdx.x; c < width; c += 256) {
     float acc = 0.f;
-    for (int q = 0; q < top; ++q) acc = fmaf(wts ? wts[t * top + q] : 1.0f, out[(static_cast<size_t>(t) * top + q) * width + c], acc);
+    for (int q = 0; q < top; ++q) {
+      float wq = wts ? wts[t * ldw + q] : 1.0f;
+      if (logits) wq = 1.0f / (1.0f + expf(-wq));
+      acc = fmaf(wq, out[(static_cast<size_t>(t) * top + q) * width + c], acc);
+    }
     x[t * ldx + c] += acc;
   }
 }
@@ -768,9 +774,11 @@ int dn_moe_down(const void* y, int y_dt, const int* order, const int* offsets, i
   return dn_launch_status();
 }
 
-int dn_moe_combine(const float* out, const float* wts, int T, int top, int width, float* x, long long ldx, hipStream_t stream) {
+int dn_moe_combine(const float* out, const float* wts, long long ldw, int logits, int T, int top, int width, float* x, long long ldx,
+                   hipStream_t stream) {
   if (T == 0) return 0;
-  hipLaunchKernelGGL(combine_kernel, dim3(T), dim3(256), 0, stream, out, wts, top, width, x, static_cast<size_t>(ldx));
+  hipLaunchKernelGGL(combine_kernel, dim3(T), dim3(256), 0, stream, out, wts, static_cast<size_t>(ldw), logits, top, width, x,
+                     static_cast<size_t>(ldx));
   return dn_launch_status();
 }
 

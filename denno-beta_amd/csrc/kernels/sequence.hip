@@ -141,6 +141,46 @@ __global__ __launch_bounds__(256) void conv_rows_kernel(const float* h, size_t l
   }
 }
 
+// The same convolution (without the row itself, then silu) over channels that are heads' vectors, a wave a vector, and for
+// the vectors of the first `n_unit` heads (of `unit_dim` channels each; the others have `rest_dim`) the vector is then
+// divided by sqrt(sum of its squares + eps) and multiplied by the head's scale: scale_a for the first n_a of them, scale_b
+// for the others.  Queries, keys and values of a recurrence leave one kernel as the recurrence reads them.
+__global__ __launch_bounds__(64) void conv_heads_kernel(const float* h, size_t ldh, const float* w, const float* hist, const int* row_start,
+                                                        const int* slots, int S, int width, int taps, int n_unit, int unit_dim, int n_a,
+                                                        float scale_a, float scale_b, float eps, int rest_dim, float* out, size_t ldo,
+                                                        size_t hist_stride) {
+  const int t = blockIdx.x, vec = blockIdx.y, lane = threadIdx.x;
+  const bool unit = vec < n_unit;
+  const int dim = unit ? unit_dim : rest_dim;
+  const int c0 = unit ? vec * unit_dim : n_unit * unit_dim + (vec - n_unit) * rest_dim;
+  float* dst = out + static_cast<size_t>(t) * ldo + c0;
+  const int s = request_of(row_start, S, t);
+  const int slot = slots[s];
+  if (slot < 0 || t >= row_start[S]) {      // a padding row: zeros
+    for (int j = lane; j < dim; j += 64) dst[j] = 0.f;
+    return;
+  }
+  const int i = t - row_start[s];
+  const float* past = hist + static_cast<size_t>(slot) * hist_stride;
+  float ss = 0.f;
+  for (int j = lane; j < dim; j += 64) {
+    const int c = c0 + j;
+    float acc = 0.f;
+    for (int q = 0; q < taps; ++q) {
+      const int src = i - taps + 1 + q;
+      const float v = src >= 0 ? h[static_cast<size_t>(row_start[s] + src) * ldh + c] : past[static_cast<size_t>(i + q) * width + c];
+      acc = fmaf(w[c * taps + q], v, acc);
+    }
+    acc = acc / (1.0f + expf(-acc));
+    ss = fmaf(acc, acc, ss);
+    dst[j] = acc;
+  }
+  if (!unit) return;
+  ss = wave_sum(ss);
+  const float f = (vec < n_a ? scale_a : scale_b) / sqrtf(ss + eps);
+  for (int j = lane; j < dim; j += 64) dst[j] *= f;      // (a lane reads back what it wrote itself)
+}
+
 // The last `keep` rows of (history ++ this step's rows) become the history.  A thread owns a channel of a request and
 // goes through the places in ascending order: place m reads the old place m + n, which it has not written yet.
 __global__ __launch_bounds__(256) void history_update_kernel(const void* h, int h_dt, size_t ldh, float* hist, const int* row_start,
@@ -204,6 +244,44 @@ __global__ __launch_bounds__(256) void rotary_kernel(const void* src, int src_dt
     } else {
       const int k = dims + (i - half);
       store_as(dst, b + k, dst_dt, load_as(src, a + k, src_dt));
+    }
+  }
+}
+
+// Up to three runs of vectors of one row turned (or only moved) in one launch, each run to a place of its own: the
+// queries, keys and values of a fused projection on their way to the attention's rows and the cache's.
+struct TurnRun {
+  void* dst;
+  int dst_dt;
+  size_t ld_dst;
+  int src_off, dst_off, dst_stride, n_vec, width, dims;      // (src_stride is the width: the vectors lie side by side)
+};
+struct TurnRuns {
+  TurnRun run[3];
+  int n;
+};
+
+__global__ __launch_bounds__(256) void rotary_runs_kernel(const void* src, int src_dt, size_t ld_src, TurnRuns runs, const int* positions,
+                                                          const float* freq) {
+  const int t = blockIdx.x;
+  const float p = static_cast<float>(positions[t]);
+  for (int r = 0; r < runs.n; ++r) {
+    const TurnRun& u = runs.run[r];
+    const int half = u.dims / 2, per = half + (u.width - u.dims);
+    for (int e = threadIdx.x; e < u.n_vec * per; e += 256) {
+      const int n = e / per, i = e % per;
+      const size_t a = static_cast<size_t>(t) * ld_src + u.src_off + static_cast<size_t>(n) * u.width;
+      const size_t b = static_cast<size_t>(t) * u.ld_dst + u.dst_off + static_cast<size_t>(n) * u.dst_stride;
+      if (i < half) {
+        const float ang = p * freq[i];
+        const float c = cosf(ang), sn = sinf(ang);
+        const float x = load_as(src, a + 2 * i, src_dt), y = load_as(src, a + 2 * i + 1, src_dt);
+        store_as(u.dst, b + 2 * i, u.dst_dt, x * c - y * sn);
+        store_as(u.dst, b + 2 * i + 1, u.dst_dt, y * c + x * sn);
+      } else {
+        const int k = u.dims + (i - half);
+        store_as(u.dst, b + k, u.dst_dt, load_as(src, a + k, src_dt));
+      }
     }
   }
 }
@@ -290,7 +368,7 @@ struct ScanArgs {
   float* state;
   size_t slot_stride;
   const int *row_start, *slots;
-  int H, dk, dv, read_after, key_from_decay;
+  int H, dk, dv, read_after, key_from_decay, beta_logits;
   float* out;
   size_t ldo;
 };
@@ -329,6 +407,7 @@ __global__ __launch_bounds__(64) void scan_kernel(ScanArgs a) {
   // 7 / 8 of a vector load where it cost four, and those loads, not the arithmetic, were what a row waited for
   float nr[VEC ? 1 : TB][NL], nk[VEC ? 1 : TB][NL], nw[VEC ? 1 : TB][NL], nv[VEC ? 1 : TB], nb[VEC ? 1 : TB];
   f32x4 r4[VEC ? NV : 1], k4[VEC ? NV : 1], w4[VEC ? NV : 1], v4;
+  auto beta_of = [&](float z) { return a.beta_logits ? 1.0f / (1.0f + expf(-z)) : z; };      // (beta given as it is, or as sigmoid's argument)
   auto fetch = [&](int t0) {
     if constexpr (VEC) {
       const f32x4 zero = {0.f, 0.f, 0.f, 0.f}, one = {1.f, 1.f, 1.f, 1.f};
@@ -340,7 +419,7 @@ __global__ __launch_bounds__(64) void scan_kernel(ScanArgs a) {
         k4[it] = (ok && !a.key_from_decay) ? *reinterpret_cast<const f32x4*>(a.k + t * a.ldk + hq * dk + i) : zero;
         w4[it] = !ok ? one : a.w_head ? one * wh : *reinterpret_cast<const f32x4*>(a.w + t * a.ldw + h * dk + i);
       }
-      if constexpr (DELTA) nb[0] = (lane < TB && t0 + lane < row1) ? a.beta[(t0 + lane) * a.ldb + h] : 0.f;
+      if constexpr (DELTA) nb[0] = (lane < TB && t0 + lane < row1) ? beta_of(a.beta[(t0 + lane) * a.ldb + h]) : 0.f;
       const int bq = lane / (CW / 4), col = j0 + (lane % (CW / 4)) * 4, t = t0 + bq;
       v4 = (lane < TB * CW / 4 && t < row1 && col < dv) ? *reinterpret_cast<const f32x4*>(a.v + t * a.ldv + h * dv + col) : zero;
     } else {
@@ -356,7 +435,7 @@ __global__ __launch_bounds__(64) void scan_kernel(ScanArgs a) {
           nk[bq][q] = (ok && !a.key_from_decay) ? a.k[t * a.ldk + hq * dk + i] : 0.f;
           nw[bq][q] = !ok ? 1.f : a.w_head ? wh : a.w[t * a.ldw + h * dk + i];
         }
-        if constexpr (DELTA) nb[bq] = row ? a.beta[t * a.ldb + h] : 0.f;
+        if constexpr (DELTA) nb[bq] = row ? beta_of(a.beta[t * a.ldb + h]) : 0.f;
         nv[bq] = (row && live) ? a.v[t * a.ldv + h * dv + j] : 0.f;
       }
     }
@@ -541,6 +620,38 @@ int dn_conv_rows(const float* h, long long ldh, const float* w, const float* his
   return dn_launch_status();
 }
 
+int dn_conv_heads(const float* h, long long ldh, const float* w, const float* hist, const int* row_start, const int* slots, int S, int T,
+                  int taps, int n_unit, int unit_dim, int n_a, float scale_a, float scale_b, float eps, int n_rest, int rest_dim,
+                  float* out, long long ldo, long long hist_stride, hipStream_t stream) {
+  const long long width = static_cast<long long>(n_unit) * unit_dim + static_cast<long long>(n_rest) * rest_dim;
+  if (taps < 1 || S < 1 || n_unit < 0 || n_rest < 0 || n_unit + n_rest < 1 || ldh < width || ldo < width || n_a < 0 || n_a > n_unit)
+    return DN_ERR_SHAPE;
+  if (T == 0) return 0;
+  hipLaunchKernelGGL(conv_heads_kernel, dim3(T, n_unit + n_rest), dim3(64), 0, stream, h, static_cast<size_t>(ldh), w, hist, row_start,
+                     slots, S, static_cast<int>(width), taps, n_unit, unit_dim, n_a, scale_a, scale_b, eps, rest_dim, out,
+                     static_cast<size_t>(ldo), static_cast<size_t>(hist_stride));
+  return dn_launch_status();
+}
+
+// runs: n x 9 numbers (dst, dst_dt, ld_dst, src_off, dst_off, dst_stride, n_vec, width, dims), n <= 3
+int dn_rotary_runs(const void* src, int src_dt, long long ld_src, const long long* runs, int n, const int* positions, const float* freq,
+                   int T, hipStream_t stream) {
+  if (!float_kind(src_dt) || n < 1 || n > 3) return n < 1 || n > 3 ? DN_ERR_SHAPE : DN_ERR_DTYPE;
+  TurnRuns r{};
+  r.n = n;
+  for (int i = 0; i < n; ++i) {
+    const long long* q = runs + 9 * i;
+    r.run[i] = TurnRun{reinterpret_cast<void*>(q[0]), static_cast<int>(q[1]), static_cast<size_t>(q[2]), static_cast<int>(q[3]),
+                       static_cast<int>(q[4]), static_cast<int>(q[5]), static_cast<int>(q[6]), static_cast<int>(q[7]),
+                       static_cast<int>(q[8])};
+    if (!float_kind(r.run[i].dst_dt)) return DN_ERR_DTYPE;
+    if (r.run[i].dims % 2 != 0 || r.run[i].dims < 0 || r.run[i].dims > r.run[i].width || r.run[i].n_vec < 0) return DN_ERR_SHAPE;
+  }
+  if (T == 0) return 0;
+  hipLaunchKernelGGL(rotary_runs_kernel, dim3(T), dim3(256), 0, stream, src, src_dt, static_cast<size_t>(ld_src), r, positions, freq);
+  return dn_launch_status();
+}
+
 int dn_history_update(const void* h, int h_dt, long long ldh, float* hist, const int* row_start, const int* slots, int S, int width,
                       int keep, long long hist_stride, hipStream_t stream) {
   if (!float_kind(h_dt)) return DN_ERR_DTYPE;
@@ -595,7 +706,7 @@ int dn_gated(const void* x, int x_dt, long long ldx, const float* g, long long l
 int dn_state_scan(const float* r, long long ldr, const float* k, long long ldk, const float* v, long long ldv, const float* w,
                   long long ldw, const float* u, const float* beta, long long ldb, const float* w_head, int G, float* state,
                   long long slot_stride, const int* row_start, const int* slots, int S, int T, int H, int dk, int dv, int mode,
-                  int key_from_decay, float* out, long long ldo, hipStream_t stream) {
+                  int key_from_decay, int beta_logits, float* out, long long ldo, hipStream_t stream) {
   if (dk < 1 || dk > 256 || dv < 1 || H < 1 || G < 1 || H % G != 0) return DN_ERR_SHAPE;
   if (!key_from_decay && k == nullptr) return DN_ERR_SHAPE;
   if (mode < SCAN_BEFORE || mode > SCAN_DELTA || (mode == SCAN_DELTA && beta == nullptr) || (w == nullptr) == (w_head == nullptr))
@@ -603,7 +714,7 @@ int dn_state_scan(const float* r, long long ldr, const float* k, long long ldk, 
   if (S == 0) return 0;
   const int read_after = mode;
   ScanArgs a{r, k, v, w, u, beta, w_head, static_cast<size_t>(ldr), static_cast<size_t>(ldk), static_cast<size_t>(ldv),
-             static_cast<size_t>(ldw), static_cast<size_t>(ldb), G, state, static_cast<size_t>(slot_stride), row_start, slots, H, dk, dv, read_after, key_from_decay, out,
+             static_cast<size_t>(ldw), static_cast<size_t>(ldb), G, state, static_cast<size_t>(slot_stride), row_start, slots, H, dk, dv, read_after, key_from_decay, beta_logits, out,
              static_cast<size_t>(ldo)};
   // (the parts of a column's sum by the head's size alone, never by the step: a row's bits are the same in every step)
   const dim3 few((dv + 15) / 16, H, S), many((dv + 3) / 4, H, S);

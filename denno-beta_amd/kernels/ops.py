@@ -130,12 +130,14 @@ def _declare(name, lib):
             "dn_unit_heads": [P, c_longlong, P, c_longlong, I, I, I, F, F, P],
             "dn_conv_rows": [P, c_longlong, P, P, P, P, I, I, I, I, I, I, P, I, c_longlong, c_longlong, P],
             "dn_history_update": [P, I, c_longlong, P, P, P, I, I, I, c_longlong, P],
+            "dn_conv_heads": [P, c_longlong, P, P, P, P, I, I, I, I, I, I, F, F, F, I, I, P, c_longlong, c_longlong, P],
+            "dn_rotary_runs": [P, I, c_longlong, P, I, P, P, I, P],
             "dn_shift_mix": [P, I, P, P, I, P, P, I, I, I, P, I, c_longlong, P],
             "dn_rotary": [P, I, c_longlong, I, I, P, I, c_longlong, I, I, P, P, I, I, I, I, P],
             "dn_activate": [P, c_longlong, P, P, I, P, I, c_longlong, I, I, P],
             "dn_gated": [P, I, c_longlong, P, c_longlong, I, P, I, c_longlong, I, I, P],
             "dn_state_scan": [P, c_longlong, P, c_longlong, P, c_longlong, P, c_longlong, P, P, c_longlong, P, I, P, c_longlong, P, P,
-                              I, I, I, I, I, I, I, P, c_longlong, P],
+                              I, I, I, I, I, I, I, I, P, c_longlong, P],
             "dn_head_norm": [P, c_longlong, P, I, F, P, c_longlong, I, P, I, c_longlong, I, I, I, P],
         },
         "grouped": {
@@ -144,7 +146,7 @@ def _declare(name, lib):
             "dn_moe_plan": [P, I, I, P, P, P],
             "dn_moe_up": [P, I, c_longlong, P, P, I, I, I, P, P, I, I, I, F, F, I, P, P, I, I, P],
             "dn_moe_down": [P, I, P, P, I, I, P, I, I, I, P, I, P],
-            "dn_moe_combine": [P, P, I, I, I, P, c_longlong, P],
+            "dn_moe_combine": [P, P, c_longlong, I, I, I, I, P, c_longlong, P],
         },
         "sampling": {
             "dn_sample": [P, I, I, I, P, P, P, P],
@@ -1034,6 +1036,48 @@ def history_update(h, hist, row_start, slots):
                                            slots.data_ptr(), S, width, keep, stride, _stream()), "history_update")
 
 
+def conv_heads(h, w, hist, row_start, slots, out, n_unit, unit_dim, n_first, scale_first, scale_rest, eps, n_rest, rest_dim):
+    """conv_rows(identity=False, act="silu") over channels that are heads' vectors, and the first n_unit vectors (unit_dim
+    channels each; n_rest more of rest_dim follow) made unit vectors on the way out: x / sqrt(sum(x^2) + eps), times
+    scale_first for the first n_first of them and scale_rest for the others.  h: 32-bit rows whose first columns are the
+    channels; out: 32-bit [T, channels]."""
+    _dev(h, "h", (torch.float32,), 2), _dev(w, "w", (torch.float32,), 2), _dev(out, "out", (torch.float32,), 2)
+    T = h.shape[0]
+    width, taps = w.shape
+    S = _request_tables(row_start, slots, "conv_heads")
+    _need(width == n_unit * unit_dim + n_rest * rest_dim and h.shape[1] >= width and w.is_contiguous() and tuple(out.shape) == (T, width)
+          and 0 <= n_first <= n_unit and n_unit + n_rest >= 1 and n_unit + n_rest <= 65535, "conv_heads: shapes")
+    stride = _history(hist, (taps - 1) * width, "conv_heads") if taps > 1 else 0
+    _ok(_lib("sequence").dn_conv_heads(h.data_ptr(), _rows(h, "h"), w.data_ptr(), _ptr(hist) if taps > 1 else 0, row_start.data_ptr(),
+                                       slots.data_ptr(), S, T, taps, n_unit, unit_dim, n_first, float(scale_first), float(scale_rest),
+                                       float(eps), n_rest, rest_dim, out.data_ptr(), _rows(out, "out"), stride, _stream()), "conv_heads")
+    return out
+
+
+def rotary_runs(src, positions, freq, runs):
+    """Up to three runs of vectors of src's rows in one launch.  runs: [(dst, src_off, n_vec, width, dims, dst_off, dst_stride)]:
+    the n_vec vectors of `width` numbers that lie side by side from column src_off go to columns dst_off + n * dst_stride of
+    dst, their first `dims` entries turned in pairs by positions[t] * freq[i] (dims 0: only moved); as `rotary` does."""
+    _dev(src, "src", _FLOATS, 2), _dev(positions, "positions", _I32, 1)
+    T = src.shape[0]
+    _need(1 <= len(runs) <= 3 and positions.is_contiguous() and positions.shape[0] == T, "rotary_runs: runs or rows")
+    table, most = [], 0
+    for dst, src_off, n_vec, width, dims, dst_off, dst_stride in runs:
+        _dev(dst, "dst", _FLOATS, 2)
+        _need(dst.shape[0] == T and dims % 2 == 0 and 0 <= dims <= width and n_vec >= 0, "rotary_runs: a run's sizes")
+        if n_vec:
+            _need(src_off >= 0 and src_off + n_vec * width <= src.shape[1] and dst_off >= 0
+                  and dst_off + (n_vec - 1) * dst_stride + width <= dst.shape[1], "rotary_runs: vectors outside their rows")
+        table += [dst.data_ptr(), _CODE[dst.dtype], _rows(dst, "dst"), src_off, dst_off, dst_stride, n_vec, width, dims]
+        most = max(most, dims)
+    _f32vec(freq, "freq")
+    _need(freq.numel() >= most // 2 and all(r[4] in (0, most) for r in runs), "rotary_runs: one table of frequencies for the turned runs")
+    import ctypes
+    arr = (ctypes.c_longlong * len(table))(*table)
+    _ok(_lib("sequence").dn_rotary_runs(src.data_ptr(), _CODE[src.dtype], _rows(src, "src"), arr, len(runs), positions.data_ptr(),
+                                        freq.data_ptr(), T, _stream()), "rotary_runs")
+
+
 def shift_mix(h, hist, mu, row_start, slots, out):
     """out[m, t, :] = h[t] + (h[t - 1] - h[t]) * mu[m]; the row before a request's first row of the step is hist[slot]."""
     _dev(h, "h", _FLOATS, 2), _dev(out, "out", _FLOATS, 3)
@@ -1093,7 +1137,7 @@ def gated(x, g, kind, out):
 
 
 def state_scan(r, k, v, w, u, state, row_start, slots, n_heads, dk, dv, out, read_after=False, key_from_decay=False, beta=None,
-               w_head=None, qk_heads=None):
+               w_head=None, qk_heads=None, beta_logits=False):
     """The recurrence of a matrix state per head, S [dk, dv], over each request's rows of this step in order:
       a = 1 - w if key_from_decay else k
       read_after:  S <- diag(w) S + a v^T ;  o = S^T r
@@ -1101,7 +1145,7 @@ def state_scan(r, k, v, w, u, state, row_start, slots, n_heads, dk, dv, out, rea
       else:        o = (S + diag(u) a v^T)^T r ;  S <- diag(w) S + a v^T        (u None: no bonus)
     r, k: 32-bit [T, qk_heads * dk] (qk_heads None: n_heads; fewer: head h reads head h // (n_heads // qk_heads));
     w: 32-bit [T, heads * dk], or None with w_head: 32-bit [heads], one decay per head for every row and channel;
-    v, out: 32-bit [T, heads * dv]; beta: 32-bit [T, heads]; state: 32-bit [slots, heads * dv * dk] (a head's state
+    v, out: 32-bit [T, heads * dv]; beta: 32-bit [T, heads] (beta_logits: it holds z, and beta is 1 / (1 + e^-z)); state: 32-bit [slots, heads * dv * dk] (a head's state
     held [value column][key channel]), read and written at the requests' slots."""
     G = n_heads if qk_heads is None else qk_heads
     _need(G >= 1 and n_heads % G == 0, lambda: f"state_scan: {n_heads} heads over {G} heads of queries and keys")
@@ -1125,7 +1169,8 @@ def state_scan(r, k, v, w, u, state, row_start, slots, n_heads, dk, dv, out, rea
                                        _rows(w, "w") if w is not None else 0, _ptr(u), _ptr(beta),
                                        _rows(beta, "beta") if beta is not None else 0, _ptr(w_head), G, state.data_ptr(), stride,
                                        row_start.data_ptr(), slots.data_ptr(), S, T, n_heads, dk, dv, mode, int(key_from_decay),
-                                       out.data_ptr(), _rows(out, "out"), _stream()), "state_scan")
+                                       int(bool(beta_logits)), out.data_ptr(), _rows(out, "out"), _stream()),
+        "state_scan" if beta is None else "state_scan (delta rule)")
     return out
 
 
@@ -1248,14 +1293,16 @@ def moe_down(y, order, offsets, w_down, out, dims=None):
                                     _CODE[wdt], width, ff, out.data_ptr(), int(dims is not None), _stream()), "moe_down")
 
 
-def moe_combine(out, wts, x):
-    """x[t, :] += sum_c wts[t, c] * out[t * top + c, :], the choices in their order (wts None: every weight is 1)."""
+def moe_combine(out, wts, x, logits=False):
+    """x[t, :] += sum_c wts[t, c] * out[t * top + c, :], the choices in their order (wts None: every weight is 1; logits: a
+    weight is 1 / (1 + e^-z) of what wts holds; wts may be columns of wider rows)."""
     _dev(out, "out", (torch.float32,), 2), _dev(x, "x", (torch.float32,), 2)
     T, width = x.shape
     top = out.shape[0] // max(T, 1) if wts is None else wts.shape[1]
     if wts is not None:
         _dev(wts, "wts", (torch.float32,), 2)
-        _need(wts.is_contiguous() and wts.shape[0] == T, "moe_combine: weights")
+        _need(wts.shape[0] == T and not (logits and wts is None), "moe_combine: weights")
     _need(out.is_contiguous() and tuple(out.shape) == (T * top, width), "moe_combine: shapes")
-    _ok(_lib("grouped").dn_moe_combine(out.data_ptr(), _ptr(wts), T, top, width, x.data_ptr(), _rows(x, "x"), _stream()),
+    _ok(_lib("grouped").dn_moe_combine(out.data_ptr(), _ptr(wts), _rows(wts, "wts") if wts is not None else 0, int(bool(logits)), T, top,
+                                       width, x.data_ptr(), _rows(x, "x"), _stream()),
         "moe_combine")

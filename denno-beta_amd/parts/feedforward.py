@@ -206,8 +206,7 @@ class RoutedExperts(Part):
             s = self.shared_down(f, out_dtype=torch.float32)
             if self.token_gate:
                 E = self.n_experts
-                share = ops.activate(z[:, E:E + 1], "sigmoid", torch.empty((T, 1), dtype=torch.float32, device=dev))
-                ops.moe_combine(s, share, accumulate_into)
+                ops.moe_combine(s, z[:, E:E + 1], accumulate_into, logits=True)      # (times sigmoid of the gate's column)
             else:
                 ops.moe_combine(s, None, accumulate_into)
         if returns:

@@ -99,15 +99,13 @@ class CausalSelfAttention(Part):
         q = new((T, H * hw), dtype=act, device=dev)
         kv = new((T, 2 * G * hw), dtype=act, device=dev)      # keys at column 0, values at G * hw
 
-        def move(n_vec, width, src_off, dst, dst_off, turn):
-            if turn:
-                position.turn(z, dst, ctx.positions, n_vec, width, src_off=src_off, src_stride=width, dst_off=dst_off, dst_stride=hw)
-            else:
-                ops.rotary(z, dst, ctx.positions, self.no_freq, n_vec, 0, width, src_off=src_off, src_stride=width, dst_off=dst_off,
-                           dst_stride=hw)
-        move(H, dk, 0, q, 0, turns)
-        move(G, dk, self.q_width, kv, 0, turns)
-        move(G, dv, self.q_width + self.kv_width, kv, G * hw, False)
+        if turns and not hasattr(position, "freq"):
+            raise TypeError(f"{type(position).__name__}: the 32-bit turn needs an encoding with a table of frequencies (rotary_pairs)")
+        dims = position.dims if turns else 0
+        freq = position.freq if turns else self.no_freq
+        # (one launch: queries and keys turned, values moved, each to its place in rows of the kept width)
+        ops.rotary_runs(z, ctx.positions, freq, [(q, 0, H, dk, dims, 0, hw), (kv, self.q_width, G, dk, dims, 0, hw),
+                                                 (kv, self.q_width + self.kv_width, G, dv, 0, G * hw, hw)])
         if cache.writes:
             ops.kv_write(kv, 0, G * hw, g.slot_map, cache.k, cache.v)
         o = torch.empty((T, H * hw), dtype=act, device=dev)

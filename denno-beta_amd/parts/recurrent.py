@@ -191,10 +191,12 @@ class ChannelDelta(Part):
         self.channels = 2 * self.qk + self.vw
         self.decay_rank, self.gate_rank = decay_rank, gate_rank
         n = names
-        # one product for everything that reads h: q | k | v | b | a1 | g1
-        self.proj = Linear(width, self.channels + n_heads + decay_rank + gate_rank, n["q"] + "+k+v+b+a1+g1", None,
-                           init_std=width ** -0.5, weight_sources=((n["q"], self.qk), (n["k"], self.qk), (n["v"], self.vw), (n["b"], n_heads),
-                                           (n["a1"], decay_rank), (n["g1"], gate_rank)))
+        # two products for everything that reads h: q | k | v | b, which stay 32-bit for the recurrence, and a1 | g1, whose
+        # results are the next products' rows
+        self.proj = Linear(width, self.channels + n_heads, n["q"] + "+k+v+b", None, init_std=width ** -0.5,
+                           weight_sources=((n["q"], self.qk), (n["k"], self.qk), (n["v"], self.vw), (n["b"], n_heads)))
+        self.low = Linear(width, decay_rank + gate_rank, n["a1"] + "+g1", None, init_std=width ** -0.5,
+                          weight_sources=((n["a1"], decay_rank), (n["g1"], gate_rank)))
         self.a2 = Linear(decay_rank, self.gw, n["a2"], None, init_std=decay_rank ** -0.5)
         self.g2 = Linear(gate_rank, self.vw, n["g2"], None, init_std=gate_rank ** -0.5)
         self.out = Linear(self.vw, width, n["o"], None)
@@ -202,7 +204,7 @@ class ChannelDelta(Part):
     def param_specs(self):
         n, taps = self.names, self.taps
         specs = []
-        for lin in (self.proj, self.a2, self.g2, self.out):
+        for lin in (self.proj, self.low, self.a2, self.g2, self.out):
             specs += lin.param_specs()
         return specs + [
             ParamSpec(n["q_conv"] + "+k+v", (self.channels, taps), "vector", ("normal", 0.0, 0.4),
@@ -216,13 +218,16 @@ class ChannelDelta(Part):
 
     def bind(self, tensors, runtime):
         super().bind(tensors, runtime)
-        for lin in (self.proj, self.a2, self.g2, self.out):
+        for lin in (self.proj, self.low, self.a2, self.g2, self.out):
             lin.bind(tensors)
         n = self.names
         self.conv = tensors[n["q_conv"] + "+k+v"]
         self.dt_bias, self.norm = tensors[n["dt_bias"]], tensors[n["norm"]]
         # the decay's rate per head, spread over the head's key channels
         self.rate = torch.exp(tensors[n["A_log"]].to(F32)).repeat_interleave(self.head_dim).contiguous()
+        # the second halves of the small products read columns of the first halves' rows where those start at 16 bytes
+        per = 16 // (2 if self.a2.weight.dtype == torch.bfloat16 else 4)
+        self._views_fit = self.decay_rank % per == 0 and (self.decay_rank + self.gate_rank) % per == 0
 
     def forward(self, h, ctx, cache, accumulate_into):
         act, T, dev = self.runtime.act_dtype, h.shape[0], h.device
@@ -231,20 +236,23 @@ class ChannelDelta(Part):
         state, past = cache.state[:, :n_state], cache.state[:, n_state:]
         z = self.proj(h, out_dtype=F32)
         x = torch.empty((T, C), dtype=F32, device=dev)
-        ops.conv_rows(z[:, :C], self.conv, past, ctx.row_start, ctx.state_slots, x, identity=False, act="silu")
+        # the three convolutions, silu, and queries and keys made unit vectors (the queries times dim^(-1/2)): one kernel
+        ops.conv_heads(z[:, :C], self.conv, past, ctx.row_start, ctx.state_slots, x, 2 * self.n_qk_heads, self.head_dim,
+                       self.n_qk_heads, self.head_dim ** -0.5, 1.0, self.UNIT_EPS, H, self.value_dim)
         if self.taps > 1 and cache.writes:
             ops.history_update(z[:, :C], past, ctx.row_start, ctx.state_slots)
         q, k, v = x[:, :qk], x[:, qk:2 * qk], x[:, 2 * qk:]
-        ops.unit_heads(q, self.n_qk_heads, self.head_dim, self.UNIT_EPS, self.head_dim ** -0.5, q)
-        ops.unit_heads(k, self.n_qk_heads, self.head_dim, self.UNIT_EPS, 1.0, k)
-        beta = ops.activate(z[:, C:C + H], "sigmoid", torch.empty((T, H), dtype=F32, device=dev))
-        low = C + H
-        g = self.a2(z[:, low:low + self.decay_rank].contiguous(), out_dtype=F32)
+        low = self.low(h, out_dtype=self.a2.weight.dtype)
+        a_in, g_in = low[:, :self.decay_rank], low[:, self.decay_rank:]
+        if not self._views_fit:      # (rows that the products cannot read where they lie)
+            a_in, g_in = a_in.contiguous(), g_in.contiguous()
+        g = self.a2(a_in, out_dtype=F32)
         ops.activate(g, "exp_neg_softplus", g, bias=self.dt_bias, lower=self.rate)
-        gate = self.g2(z[:, low + self.decay_rank:].contiguous(), out_dtype=F32)
+        gate = self.g2(g_in, out_dtype=F32)
         o = torch.empty((T, vw), dtype=F32, device=dev)
-        ops.state_scan(q, k, v, g, None, state, ctx.row_start, ctx.state_slots, H, self.head_dim, self.value_dim, o, beta=beta,
-                       qk_heads=self.n_qk_heads)
+        # (beta = sigmoid of the projection's columns behind the channels, taken inside the scan)
+        ops.state_scan(q, k, v, g, None, state, ctx.row_start, ctx.state_slots, H, self.head_dim, self.value_dim, o, beta=z[:, C:C + H],
+                       qk_heads=self.n_qk_heads, beta_logits=True)
         y = torch.empty((T, vw), dtype=act, device=dev)
         ops.head_norm(o, self.norm, self.eps, y, H, gate=gate, gate_kind="sigmoid")
         if accumulate_into is None:

@@ -304,6 +304,23 @@ def conv_rows(h, w, hist, row_start, slots, out, identity=True, act=None):
     return out
 
 
+def conv_heads(h, w, hist, row_start, slots, out, n_unit, unit_dim, n_first, scale_first, scale_rest, eps, n_rest, rest_dim):
+    conv_rows(h, w, hist, row_start, slots, out, identity=False, act="silu")
+    T = out.shape[0]
+    if n_unit:
+        v = out[:, :n_unit * unit_dim].reshape(T, n_unit, unit_dim)
+        scale = torch.cat([torch.full((n_first,), float(scale_first)), torch.full((n_unit - n_first,), float(scale_rest))])
+        y = v / torch.sqrt((v * v).sum(dim=-1, keepdim=True) + eps) * scale[None, :, None]
+        out[:, :n_unit * unit_dim] = y.reshape(T, -1)
+    return out
+
+
+def rotary_runs(src, positions, freq, runs):
+    for dst, src_off, n_vec, width, dims, dst_off, dst_stride in runs:
+        rotary(src, dst, positions, freq[:dims // 2], n_vec, dims, width, src_off=src_off, src_stride=width, dst_off=dst_off,
+               dst_stride=dst_stride)
+
+
 def history_update(h, hist, row_start, slots):
     width = h.shape[1]
     keep = hist.shape[1] // width
@@ -349,8 +366,10 @@ def gated(x, g, kind, out):
 
 
 def state_scan(r, k, v, w, u, state, row_start, slots, n_heads, dk, dv, out, read_after=False, key_from_decay=False, beta=None,
-               w_head=None, qk_heads=None):
+               w_head=None, qk_heads=None, beta_logits=False):
     H = n_heads
+    if beta is not None and beta_logits:
+        beta = torch.sigmoid(beta)
     G = H if qk_heads is None else qk_heads
     spread = lambda x: x.view(G, dk).repeat_interleave(H // G, dim=0)      # noqa: E731  (head h reads head h // (H // G))
     for slot, a, b in _requests(row_start, slots):
@@ -450,8 +469,10 @@ def moe_down(y, order, offsets, w_down, out, dims=None):
             out[int(order[p])] = w_down[e].float() @ y[p].float()
 
 
-def moe_combine(out, wts, x):
+def moe_combine(out, wts, x, logits=False):
     T = x.shape[0]
+    if logits:
+        wts = torch.sigmoid(wts)
     if wts is None:
         x += out.view(T, -1, x.shape[1]).sum(dim=1)
         return

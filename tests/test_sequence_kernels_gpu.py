@@ -173,6 +173,61 @@ def test_conv_without_the_row_itself_then_silu(taps):
         close(mine, theirs)
 
 
+@pytest.mark.parametrize("taps", [1, 3, 4])
+@pytest.mark.parametrize("n_unit,unit_dim,n_rest,rest_dim", [(4, 8, 3, 12), (2, 70, 1, 300), (6, 5, 0, 1), (0, 1, 2, 9)])
+def test_conv_of_heads_with_unit_vectors(taps, n_unit, unit_dim, n_rest, rest_dim):
+    width = n_unit * unit_dim + n_rest * rest_dim
+    row_start, slots, T = tables([1, 7, 2, 3], [2, 0, -1, 3])
+    h = torch.randn(T, width + 5, device=DEV)
+    w = torch.randn(width, taps, device=DEV)
+    hist = torch.randn(5, max(taps - 1, 1) * width + 2, device=DEV)[:, 2:2 + (taps - 1) * width]
+    both("conv_heads", lambda: (h[:, :width], w, hist, row_start, slots, torch.zeros(T, width, device=DEV), n_unit, unit_dim, n_unit // 2,
+                                unit_dim ** -0.5, 1.0, 1e-6, n_rest, rest_dim), [5])
+
+
+@pytest.mark.parametrize("dtype", DT)
+def test_three_runs_turned_in_one_launch(dtype):
+    T, H, G, dk, dv, hw, dims = 9, 4, 2, 12, 20, 32, 8
+    z = torch.randn(T, H * dk + G * dk + G * dv, device=DEV)
+    positions = torch.randint(0, 500, (T,), dtype=torch.int32, device=DEV)
+    freq = torch.rand(dims // 2, device=DEV)
+
+    def make():
+        q, kv = torch.zeros(T, H * hw, dtype=dtype, device=DEV), torch.zeros(T, 2 * G * hw, dtype=dtype, device=DEV)
+        return (z, positions, freq, [(q, 0, H, dk, dims, 0, hw), (kv, H * dk, G, dk, dims, 0, hw), (kv, H * dk + G * dk, G, dv, 0, G * hw, hw)])
+    args = make()
+    host = [z.cpu(), positions.cpu(), freq.cpu(), [(torch.zeros_like(r[0]).cpu(),) + r[1:] for r in args[3]]]
+    host[3][2] = (host[3][1][0],) + host[3][2][1:]          # (keys and values share their rows)
+    ops.rotary_runs(*args)
+    ref.rotary_runs(*host)
+    close(args[3][0][0], host[3][0][0], dtype, "queries")
+    close(args[3][1][0], host[3][1][0], dtype, "keys and values")
+
+
+def test_delta_rule_with_beta_as_sigmoid_argument():
+    row_start, slots, T = tables([5, 1], [1, 0])
+    H, dk, dv = 2, 16, 8
+    r, k, v, w = (torch.randn(T, H * n, device=DEV) for n in (dk, dk, dv, dk))
+    w = torch.sigmoid(w)
+    z = torch.randn(T, H + 3, device=DEV)
+    state = torch.randn(2, H * dk * dv, device=DEV)
+    a = ops.state_scan(r, k, v, w, None, state.clone(), row_start, slots, H, dk, dv, torch.zeros(T, H * dv, device=DEV), beta=z[:, 1:1 + H],
+                       beta_logits=True)
+    b = ops.state_scan(r, k, v, w, None, state.clone(), row_start, slots, H, dk, dv, torch.zeros(T, H * dv, device=DEV),
+                       beta=torch.sigmoid(z[:, 1:1 + H]).contiguous())
+    close(a, b)
+
+
+def test_sum_of_results_weighted_by_sigmoid_of_a_column():
+    T, width = 7, 40
+    out, x = torch.randn(T, width, device=DEV), torch.randn(T, width, device=DEV)
+    z = torch.randn(T, 6, device=DEV)
+    hx = x.cpu().clone()
+    ops.moe_combine(out, z[:, 5:6], x, logits=True)
+    ref.moe_combine(out.cpu(), z[:, 5:6].cpu(), hx, logits=True)
+    close(x, hx)
+
+
 @pytest.mark.parametrize("width", [7, 96, 1000])
 @pytest.mark.parametrize("dtype", DT)
 def test_norm_added_into_the_stream(width, dtype):
