@@ -555,6 +555,26 @@ __global__ __launch_bounds__(64) void head_norm_kernel(const float* o, size_t ld
   }
 }
 
+// The same for heads of many columns (all heads normed as one vector): a workgroup a head, the sums as in rmsnorm_kernel.
+// Which of the two kernels runs depends on the head's size alone.
+__global__ __launch_bounds__(256) void head_norm_wide_kernel(const float* o, size_t ld, const float* weight, int w_stride, float eps,
+                                                             const float* gate, size_t ldg, int gate_kind, void* out, int out_dt,
+                                                             size_t ldo, int dv) {
+  __shared__ float sh[4];
+  const int t = blockIdx.x, h = blockIdx.y;
+  const float* src = o + t * ld + static_cast<size_t>(h) * dv;
+  float ss = 0.f;
+  for (int j = threadIdx.x; j < dv; j += 256) ss = fmaf(src[j], src[j], ss);
+  ss = block_sum_256(ss, sh);
+  const float inv = 1.0f / sqrtf(ss / static_cast<float>(dv) + eps);
+  for (int j = threadIdx.x; j < dv; j += 256) {
+    float y = src[j] * inv;
+    if (weight) y *= weight[h * w_stride + j];
+    if (gate) y *= activation(gate_kind, gate[t * ldg + static_cast<size_t>(h) * dv + j], 0.f);
+    store_as(out, t * ldo + static_cast<size_t>(h) * dv + j, out_dt, y);
+  }
+}
+
 bool float_kind(int dt) { return dt == DN_F32 || dt == DN_BF16; }
 
 }  // namespace
@@ -754,8 +774,12 @@ int dn_head_norm(const float* o, long long ld, const float* weight, int w_stride
   if (!float_kind(out_dt)) return DN_ERR_DTYPE;
   if (gate && (gate_kind < 0 || gate_kind > ACT_TANH)) return DN_ERR_SHAPE;
   if (T == 0) return 0;
-  hipLaunchKernelGGL(head_norm_kernel, dim3(T, H), dim3(64), 0, stream, o, static_cast<size_t>(ld), weight, w_stride, eps, gate,
-                     static_cast<size_t>(ldg), gate_kind, out, out_dt, static_cast<size_t>(ldo), dv);
+  if (dv > 256)
+    hipLaunchKernelGGL(head_norm_wide_kernel, dim3(T, H), dim3(256), 0, stream, o, static_cast<size_t>(ld), weight, w_stride, eps, gate,
+                       static_cast<size_t>(ldg), gate_kind, out, out_dt, static_cast<size_t>(ldo), dv);
+  else
+    hipLaunchKernelGGL(head_norm_kernel, dim3(T, H), dim3(64), 0, stream, o, static_cast<size_t>(ld), weight, w_stride, eps, gate,
+                       static_cast<size_t>(ldg), gate_kind, out, out_dt, static_cast<size_t>(ldo), dv);
   return dn_launch_status();
 }
 

@@ -312,6 +312,11 @@ def test_head_norm(dtype):
     both("head_norm", lambda: (o, torch.randn(H * dv, device=DEV), 1e-5, torch.empty(T, H * dv, dtype=dtype, device=DEV), H, gate, "silu"), [3], dtype)
     both("head_norm", lambda: (o, torch.randn(dv, device=DEV), 1e-5, torch.empty(T, H * dv, dtype=dtype, device=DEV), H), [3], dtype)
     both("head_norm", lambda: (o, None, 1e-2, torch.empty(T, H * dv, dtype=dtype, device=DEV), H), [3], dtype)
+    # all heads as one vector, and heads of many columns (a workgroup a head)
+    both("head_norm", lambda: (o, torch.randn(H * dv, device=DEV), 1e-5, torch.empty(T, H * dv, dtype=dtype, device=DEV), 1, gate, "sigmoid"), [3], dtype)
+    wide, wgate = torch.randn(T, 2 * 700, device=DEV), torch.randn(T, 2 * 700, device=DEV)
+    both("head_norm", lambda: (wide, torch.randn(700, device=DEV), 1e-5, torch.empty(T, 1400, dtype=dtype, device=DEV), 2, wgate, "sigmoid"), [3], dtype)
+    both("head_norm", lambda: (wide, torch.randn(1400, device=DEV), 1e-5, torch.empty(T, 1400, dtype=dtype, device=DEV), 1, wgate, "silu"), [3], dtype)
 
 
 @pytest.mark.parametrize("dtype", DT)
