@@ -176,17 +176,20 @@ class ChannelDelta(Part):
     graph_safe = True
     returns_rows = True
     libraries = ("sequence",)
-    UNIT_EPS = 1e-6
 
     def __init__(self, width: int, n_heads: int, n_qk_heads: int, head_dim: int, value_dim: int, taps: int, eps: float,
-                 decay_rank: int, gate_rank: int, names: dict):
-        """names: q, k, v, b, a1, a2, g1, g2, o (matrices); q_conv, k_conv, v_conv ([channels, taps]); A_log, dt_bias, norm."""
+                 decay_rank: int, gate_rank: int, names: dict, unit_eps: float = 1e-6, query_scale=None):
+        """names: q, k, v, b, a1, a2, g1, g2, o (matrices); q_conv, k_conv, v_conv ([channels, taps]); A_log, dt_bias, norm.
+        unit_eps: what is added to the sum of squares under the unit vectors' root; query_scale: what the unit queries are
+        multiplied by (None: head_dim^(-1/2))."""
         if n_heads % n_qk_heads != 0:
             raise ValueError(f"channel_delta: {n_heads} heads cannot share {n_qk_heads} heads of queries and keys")
         if taps < 1:
             raise ValueError(f"channel_delta: {taps} taps")
         self.width, self.n_heads, self.n_qk_heads, self.head_dim, self.value_dim = width, n_heads, n_qk_heads, head_dim, value_dim
         self.taps, self.eps, self.names = taps, eps, dict(names)
+        self.unit_eps = float(unit_eps)
+        self.query_scale = head_dim ** -0.5 if query_scale is None else float(query_scale)
         self.qk, self.vw, self.gw = n_qk_heads * head_dim, n_heads * value_dim, n_heads * head_dim
         self.channels = 2 * self.qk + self.vw
         self.decay_rank, self.gate_rank = decay_rank, gate_rank
@@ -238,7 +241,7 @@ class ChannelDelta(Part):
         x = torch.empty((T, C), dtype=F32, device=dev)
         # the three convolutions, silu, and queries and keys made unit vectors (the queries times dim^(-1/2)): one kernel
         ops.conv_heads(z[:, :C], self.conv, past, ctx.row_start, ctx.state_slots, x, 2 * self.n_qk_heads, self.head_dim,
-                       self.n_qk_heads, self.head_dim ** -0.5, 1.0, self.UNIT_EPS, H, self.value_dim)
+                       self.n_qk_heads, self.query_scale, 1.0, self.unit_eps, H, self.value_dim)
         if self.taps > 1 and cache.writes:
             ops.history_update(z[:, :C], past, ctx.row_start, ctx.state_slots)
         q, k, v = x[:, :qk], x[:, qk:2 * qk], x[:, 2 * qk:]
